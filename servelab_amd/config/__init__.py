@@ -2,6 +2,7 @@ from .model import ConfigError, Qwen2Config, read_key
 from .layered import (BiasedAttentionConfig, DenseMlpConfig, LatentAttentionConfig, LayerConfig,
                       TopelornConfig, WindowConfig)
 from .vekanex import VekanexConfig, VekanexLayer
+from .futezen import FutezenConfig, FutezenLayer
 from .engine import CacheConfig, SchedulerConfig, EngineConfig, PAGE_SIZES
 from .registry import (Architecture, register_architecture, registered_architectures,
                        resolve_architecture)

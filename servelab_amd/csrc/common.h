@@ -51,6 +51,14 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return t;
 }
 
+// Activations by number, as the calls of the kernel table pass them: 1 silu, 2 relu, 3 relu squared.
+enum { SL_ACT_SILU = 1, SL_ACT_RELU = 2, SL_ACT_RELU2 = 3 };
+__device__ __forceinline__ float sl_act(float z, int act) {
+  if (act == SL_ACT_SILU) return z / (1.f + expf(-z));
+  const float r = fmaxf(z, 0.f);
+  return act == SL_ACT_RELU2 ? r * r : r;
+}
+
 #define SL_CHECK(cond, msg) \
   do { if (!(cond)) return msg; } while (0)
 

@@ -27,8 +27,9 @@ extern "C" const char* sl_embed(const int* ids, const void* table, float* out, i
 // (servelab/parallel/tp_model.py:68), float inside.  A row of gate_up holds
 // gate and up interleaved in blocks: gate i sits at 2 * block * (i / block) +
 // i % block and up i one block further; block = I is plain [gate | up].
+// `act` names another activation of the gate than silu (common.h).
 __global__ void silu_mul_kernel(const act_t* __restrict__ gate_up, act_t* __restrict__ out,
-                                int I, int block, size_t total) {
+                                int I, int block, size_t total, int act) {
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (size_t)gridDim.x * blockDim.x) {
     const size_t t = idx / I;
@@ -36,7 +37,7 @@ __global__ void silu_mul_kernel(const act_t* __restrict__ gate_up, act_t* __rest
     const size_t at = t * 2 * I + (size_t)2 * block * (i / block) + i % block;
     const float g = to_f(gate_up[at]);
     const float u = to_f(gate_up[at + block]);
-    out[idx] = from_f<act_t>(g / (1.f + expf(-g)) * u);
+    out[idx] = from_f<act_t>(sl_act(g, act) * u);
   }
 }
 
@@ -75,13 +76,14 @@ __global__ void silu_mul_block8_kernel(const act_t* __restrict__ gate_up, act_t*
   }
 }
 
-extern "C" const char* sl_silu_mul(const void* gate_up, void* out, int T, int I, int block,
+extern "C" const char* sl_gate_mul(const void* gate_up, void* out, int T, int I, int block, int act,
                                    hipStream_t stream) {
   SL_CHECK(T >= 0 && I > 0, "silu_mul: sizes must be positive");
+  SL_CHECK(act >= SL_ACT_SILU && act <= SL_ACT_RELU2, "gate_mul: unknown activation");
   SL_CHECK(block > 0 && I % block == 0, "silu_mul: the block must divide the width");
   if (T == 0) return nullptr;
   const size_t total = (size_t)T * I;
-  if (block == 8 && ((uintptr_t)gate_up % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+  if (act == SL_ACT_SILU && block == 8 && ((uintptr_t)gate_up % 16) == 0 && ((uintptr_t)out % 16) == 0) {
     const size_t groups = total / 8;
     const size_t blocks = (groups + 255) / 256;
     silu_mul_block8_kernel<<<(unsigned)(blocks < 262144 ? blocks : 262144), 256, 0, stream>>>(
@@ -89,7 +91,28 @@ extern "C" const char* sl_silu_mul(const void* gate_up, void* out, int T, int I,
     return sl_launch_status();
   }
   const int blocks = (int)((total + 255) / 256 < 65535 * 4 ? (total + 255) / 256 : 65535 * 4);
-  silu_mul_kernel<<<blocks, 256, 0, stream>>>((const act_t*)gate_up, (act_t*)out, I, block, total);
+  silu_mul_kernel<<<blocks, 256, 0, stream>>>((const act_t*)gate_up, (act_t*)out, I, block, total, act);
+  return sl_launch_status();
+}
+
+extern "C" const char* sl_silu_mul(const void* gate_up, void* out, int T, int I, int block,
+                                   hipStream_t stream) {
+  return sl_gate_mul(gate_up, out, T, I, block, SL_ACT_SILU, stream);
+}
+
+// out[i] = act(x[i]) (common.h's activations), float inside; out may be x.
+__global__ void activate_kernel(const act_t* __restrict__ x, act_t* __restrict__ out, size_t n, int act) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    out[i] = from_f<act_t>(sl_act(to_f(x[i]), act));
+}
+
+extern "C" const char* sl_activate(const void* x, void* out, long long n, int act, hipStream_t stream) {
+  SL_CHECK(n >= 0, "activate: the count must not be negative");
+  SL_CHECK(act >= SL_ACT_SILU && act <= SL_ACT_RELU2, "activate: unknown activation");
+  if (n == 0) return nullptr;
+  const size_t blocks = ((size_t)n + 255) / 256;
+  activate_kernel<<<(unsigned)(blocks < 262144 ? blocks : 262144), 256, 0, stream>>>((const act_t*)x, (act_t*)out,
+                                                                                     (size_t)n, act);
   return sl_launch_status();
 }
 

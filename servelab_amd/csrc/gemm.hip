@@ -476,6 +476,7 @@ struct NormFusion {
   // that do (N = 5120 on 256 CUs: 512 tiles of 10 rows instead of 320 of 16).  Other forms: 16.
   int th;
   int pair_x;                // at most 8 rows and one tile a workgroup: a load of x takes two k-steps (see stream_k2)
+  int gate_act;              // gated forms: the activation of the gate (common.h: 1 silu, 2 relu)
 };
 
 // Rotary embedding and the write to the cache pages fused into the q/k/v
@@ -743,7 +744,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
             usum *= inv;
           }
           const size_t at = F.y_tiled ? (size_t)(n / 32) * (M * 32) + m * 32 + n % 32 : (size_t)m * (N / 2) + n;
-          ((__bf16*)y)[at] = (__bf16)(gsum / (1.f + expf(-gsum)) * usum);
+          ((__bf16*)y)[at] = (__bf16)(sl_act(gsum, F.gate_act) * usum);
         }
       }
       continue;
@@ -842,7 +843,7 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
            "gemm_skinny: x tiled by k-step has as many rows as the product, or rows are picked from it");
   SL_CHECK(!y_tiled || (gated && (N / 2) % 32 == 0) || (resid != nullptr && N % 32 == 0),
            "gemm_skinny: a tiled result is a gated one or a producer's, of a multiple of 32 columns");
-  const NormFusion F{in_parts, in_nparts, eps, rows, resid, next_w, out_parts, x_tiled, y_tiled, th, pair_x};
+  const NormFusion F{in_parts, in_nparts, eps, rows, resid, next_w, out_parts, x_tiled, y_tiled, th, pair_x, gated};
   const bool few = in_nparts <= 32 * 8;
   if (rope != nullptr) {
     const RopeStore R = *rope;
@@ -985,7 +986,7 @@ __global__ __launch_bounds__(512) void gemm_resident_kernel(
           gsum *= inv;
           usum *= inv;
           const size_t at = F.y_tiled ? (size_t)(col / 32) * (M * 32) + m * 32 + col % 32 : (size_t)m * (N / 2) + col;
-          ((__bf16*)y)[at] = (__bf16)(gsum / (1.f + expf(-gsum)) * usum);
+          ((__bf16*)y)[at] = (__bf16)(sl_act(gsum, F.gate_act) * usum);
         }
       }
     } else if (threadIdx.x < 256) {
@@ -1054,7 +1055,7 @@ extern "C" const char* sl_gemm_resident(const void* x, const void* wt, const flo
   SL_CHECK(!y_tiled || (gated && (N / 2) % 32 == 0), "gemm_resident: a tiled result is a gated one of a multiple of 32 columns");
   SL_CHECK(x_tiled >= 0 && (x_tiled == 0 || rows != nullptr || x_tiled == M),
            "gemm_resident: x tiled by k-step has as many rows as the product, or rows are picked from it");
-  const NormFusion F{in_parts, in_nparts, eps, rows, nullptr, nullptr, nullptr, x_tiled, y_tiled};
+  const NormFusion F{in_parts, in_nparts, eps, rows, nullptr, nullptr, nullptr, x_tiled, y_tiled, 0, 0, gated};
   const __bf16* xx = (const __bf16*)x;
   const __bf16* ww = (const __bf16*)wt;
 #define SL_RESIDENT(G, NS, R)                                                                   \
@@ -1090,7 +1091,7 @@ extern "C" const char* sl_gemm_resident(const void* x, const void* wt, const flo
 template <int MB, bool GATED>
 __global__ __launch_bounds__(512) void gemm_wide_kernel(
     const __bf16* __restrict__ x, const __bf16* __restrict__ wt, const float* __restrict__ bias,
-    void* __restrict__ y, int M, int N, int K, int out_f32) {
+    void* __restrict__ y, int M, int N, int K, int out_f32, int gate_act) {
   constexpr int WAVES = 8, U = 2, NT = 2;
   __shared__ f32x4 red[WAVES][MB][64];
   // the wavefront's index as a scalar: what depends on it (its share of K, its tiles) then steers
@@ -1208,7 +1209,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(
             gsum += red[wv][b][m_local + 16 * (j / 4)][j % 4];
             usum += red[wv][b][m_local + 16 * (2 + j / 4)][j % 4];
           }
-          ((__bf16*)y)[(size_t)m * (N / 2) + n] = (__bf16)(gsum / (1.f + expf(-gsum)) * usum);
+          ((__bf16*)y)[(size_t)m * (N / 2) + n] = (__bf16)(sl_act(gsum, gate_act) * usum);
         }
       }
       continue;
@@ -1242,11 +1243,11 @@ extern "C" const char* sl_gemm_wide(const void* x, const void* wt, const float* 
   const __bf16* xx = (const __bf16*)x;
   const __bf16* ww = (const __bf16*)wt;
   if (gated) {
-    if (M <= 32) gemm_wide_kernel<2, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0);
-    else gemm_wide_kernel<4, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0);
+    if (M <= 32) gemm_wide_kernel<2, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, gated);
+    else gemm_wide_kernel<4, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, gated);
   } else {
-    if (M <= 32) gemm_wide_kernel<2, false><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
-    else gemm_wide_kernel<4, false><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
+    if (M <= 32) gemm_wide_kernel<2, false><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32, 0);
+    else gemm_wide_kernel<4, false><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32, 0);
   }
   return sl_launch_status();
 }
@@ -1479,7 +1480,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const float g = acc[t][b][r];
-            o[r] = (__bf16)(g / (1.f + expf(-g)) * up[r]);
+            o[r] = (__bf16)(sl_act(g, gated) * up[r]);
           }
         }
         continue;

@@ -349,6 +349,74 @@ extern "C" const char* sl_add_postnorm(float* resid, const void* y, const float*
   return sl_launch_status();
 }
 
+// A sublayer's output joins the stream through a norm of its own, and the next sublayer's input norm
+// follows at once: v = resid + y * rsqrt(mean(y^2) + eps_y) * wy, out = v * rsqrt(mean(v^2) + eps) * w.
+// rows == nullptr: every row, and v goes back to the stream; else only the listed rows are computed
+// and the stream stays as it is (the head reads few rows of the last layer's result).  One block per
+// row, up to NORMED_KEEP values a thread kept in registers between the passes; all sums in float.
+constexpr int NORMED_KEEP = 8;
+__global__ void add_normed_rmsnorm_kernel(float* __restrict__ resid, const act_t* __restrict__ y,
+                                          const float* __restrict__ wy, float eps_y,
+                                          const int* __restrict__ rows, const float* __restrict__ w, float eps,
+                                          act_t* __restrict__ out, int H) {
+  __shared__ float scratch[16];
+  const size_t r = rows != nullptr ? (size_t)rows[blockIdx.x] : (size_t)blockIdx.x;
+  float* x = resid + r * H;
+  const act_t* yr = y + r * H;
+  act_t* o = out + (size_t)blockIdx.x * H;
+  float keep[NORMED_KEEP];
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < NORMED_KEEP; ++u) {
+    const int i = threadIdx.x + u * blockDim.x;
+    keep[u] = i < H ? to_f(yr[i]) : 0.f;
+    ss += keep[u] * keep[u];
+  }
+  for (int i = threadIdx.x + NORMED_KEEP * blockDim.x; i < H; i += blockDim.x) {
+    const float v = to_f(yr[i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv_y = 1.f / sqrtf(ss / (float)H + eps_y);
+  float s2 = 0.f;
+#pragma unroll
+  for (int u = 0; u < NORMED_KEEP; ++u) {
+    const int i = threadIdx.x + u * blockDim.x;
+    if (i < H) {
+      keep[u] = x[i] + keep[u] * inv_y * wy[i];
+      if (rows == nullptr) x[i] = keep[u];
+      s2 += keep[u] * keep[u];
+    }
+  }
+  for (int i = threadIdx.x + NORMED_KEEP * blockDim.x; i < H; i += blockDim.x) {
+    const float v = x[i] + to_f(yr[i]) * inv_y * wy[i];
+    if (rows == nullptr) x[i] = v;
+    s2 += v * v;
+  }
+  s2 = block_sum(s2, scratch);
+  const float inv = 1.f / sqrtf(s2 / (float)H + eps);
+#pragma unroll
+  for (int u = 0; u < NORMED_KEEP; ++u) {
+    const int i = threadIdx.x + u * blockDim.x;
+    if (i < H) o[i] = from_f<act_t>(keep[u] * inv * w[i]);
+  }
+  for (int i = threadIdx.x + NORMED_KEEP * blockDim.x; i < H; i += blockDim.x) {
+    const float v = rows == nullptr ? x[i] : x[i] + to_f(yr[i]) * inv_y * wy[i];
+    o[i] = from_f<act_t>(v * inv * w[i]);
+  }
+}
+
+extern "C" const char* sl_add_normed_rmsnorm(float* resid, const void* y, const float* wy, float eps_y,
+                                             const int* rows, const float* w, float eps, void* out, int R,
+                                             int H, hipStream_t stream) {
+  SL_CHECK(R >= 0 && H > 0, "add_normed_rmsnorm: sizes must be positive");
+  SL_CHECK(y != nullptr && wy != nullptr && w != nullptr, "add_normed_rmsnorm: the output and both gains are required");
+  if (R == 0) return nullptr;
+  add_normed_rmsnorm_kernel<<<R, H >= 2048 ? 512 : 256, 0, stream>>>(resid, (const act_t*)y, wy, eps_y, rows, w,
+                                                                    eps, (act_t*)out, H);
+  return sl_launch_status();
+}
+
 // out = sa * a + sb * b, float sums: the outputs of two mixers that ran side by side.
 __global__ void scaled_sum_kernel(const act_t* __restrict__ a, float sa, const act_t* __restrict__ b, float sb,
                                   act_t* __restrict__ out, size_t n) {

@@ -3,11 +3,13 @@
 //
 //   lowrank_expand   z = t W2^T + b from the few columns a low-rank projection left, as a log
 //                    decay (logsigmoid(z) / tau, or -exp(rate_h) softplus(z)) or plain
-//   short_conv       silu of a causal convolution over time per channel, the last taps - 1
-//                    inputs kept in the state slot; heads made unit vectors
+//   short_conv       silu of a causal convolution over time per channel (with or without a bias),
+//                    the last taps - 1 inputs kept in the state slot; heads made unit vectors
 //   matrix_scan      the recurrences: decay per key channel (S' = diag(a) S + k v^T), the same
-//                    with the delta rule's correction (u = beta (v - S'^T k)), and the matrix
-//                    LSTM (scalar gates with a running maximum, a normaliser n)
+//                    with the delta rule's correction (u = beta (v - S'^T k)), the matrix
+//                    LSTM (scalar gates with a running maximum, a normaliser n), and the
+//                    state-space form (a scalar decay per head from a step size dt, the input
+//                    times dt, a skip of the token's own input)
 //   head_norm_gate   a head's read-out divided by its root mean square, gain, output gate
 //   projnorm_rope_store  softmax attention's q and k normed over the whole projection, rotated,
 //                    k and v written to their pages
@@ -88,6 +90,7 @@ struct ShortConv {
   const float* buf;          // inputs of token t at buf + t * stride + col
   int stride, col, C, taps;
   const float* w;            // [C][taps], the last tap is the token's own
+  const float* bias;         // [C] added before the silu, or nullptr
   float* state;              // slot s at state + s * state_stride + state_off: [taps - 1][C], oldest first
   long long state_stride;
   int state_off;
@@ -124,7 +127,7 @@ __global__ __launch_bounds__(64) void short_conv_kernel(const ShortConv a) {
     const int c = c0 + lane + u * 64;
     y[u] = 0.f;
     if (lane + u * 64 < n) {
-      float acc = 0.f;
+      float acc = a.bias != nullptr ? a.bias[c] : 0.f;
       for (int j = 0; j < a.taps; ++j) {
         const int idx = i - back + j;                       // place in the step of the tap's input
         float x;
@@ -168,7 +171,7 @@ __global__ void short_conv_state_kernel(const ShortConv a, int S) {
 }
 
 extern "C" const char* sl_short_conv(const float* buf, int stride, int col, int C, int taps, const float* w,
-                                     float* state, long long state_stride, int state_off, const int* cu_q,
+                                     const float* bias, float* state, long long state_stride, int state_off, const int* cu_q,
                                      const int* positions, const int* tok_seq, const int* slots, int S, int T,
                                      int write, int unit_heads, int unit_dim, float unit_eps, int scaled_heads,
                                      float scale, float* out, hipStream_t stream) {
@@ -180,7 +183,7 @@ extern "C" const char* sl_short_conv(const float* buf, int stride, int col, int 
   SL_CHECK(state_off >= 0 && state_off + (long long)(taps - 1) * C <= state_stride,
            "short_conv: the last inputs do not fit the state slot");
   if (T == 0) return nullptr;
-  const ShortConv a{buf, stride, col, C, taps, w, state, state_stride, state_off, cu_q, positions, tok_seq,
+  const ShortConv a{buf, stride, col, C, taps, w, bias, state, state_stride, state_off, cu_q, positions, tok_seq,
                     slots, unit_heads, unit_dim, scaled_heads, unit_eps, scale, out};
   const int rest = C - unit_heads * unit_dim;
   short_conv_kernel<<<dim3(T, unit_heads + (rest + 255) / 256), 64, 0, stream>>>(a);
@@ -196,7 +199,11 @@ struct MatrixScan {
   const float* log_decay;    // [T][H][D] (decay and delta modes)
   float q_scale;
   const float* gates;        // delta: beta before its sigmoid at gates + t * gate_stride + beta_col + h;
-  int gate_stride, i_col, f_col;   // matrix LSTM: the two gates before cap and squashing at i_col + h, f_col + h
+  int gate_stride, i_col, f_col;   // matrix LSTM: the two gates before cap and squashing at i_col + h, f_col + h;
+                             // state-space: the step size before its bias and softplus at i_col + h
+  const float* rates;        // state-space, per head: dt = softplus(raw + step_bias[h]), the state keeps
+  const float* step_bias;    // exp(-exp(rates[h]) dt) of itself and takes dt k v^T; the read-out adds
+  const float* skip;         // skip[h] v
   float cap;
   float* state;              // slot s at state + s * state_stride: S [H][Dv][D]; matrix LSTM: then n [H][D], m [H]
   long long state_stride;
@@ -207,7 +214,7 @@ struct MatrixScan {
   float* out;                // [T][H][Dv]
 };
 
-enum { SCAN_DECAY = 0, SCAN_DELTA = 1, SCAN_LSTM = 2 };
+enum { SCAN_DECAY = 0, SCAN_DELTA = 1, SCAN_LSTM = 2, SCAN_SSD = 3 };
 constexpr int SCAN_ROWS = 8;      // key channels a lane owns: channels 8 p .. 8 p + 7
 
 // Sum over the P lanes that share a column (P a power of two, the lanes adjacent and aligned); every
@@ -252,10 +259,11 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
   // The matrix LSTM's normaliser n is one more column of S whose value channel is always 1: the last
   // column group of every block carries it (every block the same one) and leaves max(|n . q|, e^-m) +
   // 1e-6 where the others leave their read-outs; these are divided by it when they leave LDS.
+  constexpr bool SCALAR = MODE == SCAN_LSTM || MODE == SCAN_SSD;      // one decay a head: no decays per channel in LDS
   const int vcols = MODE == SCAN_LSTM ? cols - 1 : cols;
-  const int half = CH * ((MODE == SCAN_LSTM ? 2 : 3) * Dp + 2 * cols + 4);
+  const int half = CH * ((SCALAR ? 2 : 3) * Dp + 2 * cols + 4);
   const int oq = 0, ok = CH * Dp, oa = 2 * CH * Dp;          // [CH][Dp] each (no decays for the matrix LSTM)
-  const int ov = MODE == SCAN_LSTM ? oa : oa + CH * Dp;       // [CH][cols]
+  const int ov = SCALAR ? oa : oa + CH * Dp;                  // [CH][cols]
   const int og = ov + CH * cols;                              // [CH][4] gates
   const int oo = og + CH * 4;                                 // [CH][cols] the walkers' read-outs
   const int g = h / (a.H / a.G);
@@ -286,7 +294,7 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
           if (r < a.D) {
             pq[e] = a.src[t * a.src_stride + a.q_col + g * a.D + r] * a.q_scale;
             pk[e] = a.src[t * a.src_stride + a.k_col + g * a.D + r];
-            if (MODE != SCAN_LSTM) pd[e] = a.log_decay[(t * a.H + h) * a.D + r];
+            if (!SCALAR) pd[e] = a.log_decay[(t * a.H + h) * a.D + r];
           }
         }
         if (idx < nt * cols) {
@@ -331,11 +339,16 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
             const int at = (idx - r) + ((r & (ROWS - 1)) >> 2) * 4 * P + (r / ROWS) * 4 + (r & 3);
             base[oq + at] = pq[e];
             base[ok + at] = pk[e];
-            if (MODE != SCAN_LSTM) base[oa + at] = expf(pd[e]);
+            if (!SCALAR) base[oa + at] = expf(pd[e]);
           }
           if (idx < nt * cols) base[ov + idx] = pv[e];
         }
         if (MODE == SCAN_DELTA && tid < nt) base[og + tid * 4] = sigmoidf_(g0);
+        if (MODE == SCAN_SSD && tid < nt) {
+          const float dt = softplusf_(g0 + a.step_bias[h]);
+          base[og + tid * 4] = expf(-expf(a.rates[h]) * dt);
+          base[og + tid * 4 + 1] = dt;
+        }
         if (MODE == SCAN_LSTM && tid < 64) {
           // (CH is at most 16: the chunk's gates sit in the first lanes of this wavefront)
           const float ig = a.cap * tanhf(g0 / a.cap), fg = logsigmoidf_(a.cap * tanhf(g1 / a.cap));
@@ -375,6 +388,7 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
   const bool live = is_n || j < a.Dv;
   float* col = is_n ? nrow : slot + ((size_t)h * a.Dv + (live ? j : 0)) * a.D;
   float S[ROWS];
+  const float skip_h = MODE == SCAN_SSD ? a.skip[h] : 0.f;
   const int r0 = p * ROWS;
   // (a lane's values of a column are 16-byte pieces where the slot's place allows it)
   const bool whole = live && r0 + ROWS <= a.D && ((uintptr_t)(col + r0) % 16) == 0;
@@ -412,7 +426,7 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
             q[4 * u + c2] = qv.v[c2];
             k[4 * u + c2] = kv.v[c2];
           }
-          if (MODE != SCAN_LSTM) {
+          if (!SCALAR) {
             const scan_f4 dv = d4[u * P];
 #pragma unroll
             for (int c2 = 0; c2 < 4; ++c2) d[4 * u + c2] = dv.v[c2];
@@ -452,6 +466,7 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
       float o = group_sum(rows_sum<ROWS>(part), P);
       // (the column that carries n leaves the divisor of its token's read-outs)
       if (MODE == SCAN_LSTM && is_n) o = fmaxf(fabsf(o), sg[tt * 4 + 2]) + 1e-6f;
+      if (MODE == SCAN_SSD) o += skip_h * v;
       if (p == 0) so[tt * cols + cl] = o;
     }
     __syncthreads();                      // chunk c + 1 is in LDS, chunk c's half is free
@@ -477,14 +492,16 @@ __global__ __launch_bounds__(512) void matrix_scan_kernel(const MatrixScan a, in
 extern "C" const char* sl_matrix_scan(int mode, const float* src, int src_stride, int q_col, int k_col, int v_col,
                                       int H, int G, int D, int Dv, const float* log_decay, float q_scale,
                                       const float* gates, int gate_stride, int i_col, int f_col, float cap,
-                                      float* state, long long state_stride, const int* cu_q, const int* positions,
+                                      const float* rates, const float* step_bias, const float* skip, float* state, long long state_stride, const int* cu_q, const int* positions,
                                       const int* slots, int S, int T, int write, float* out, hipStream_t stream) {
-  SL_CHECK(mode >= 0 && mode <= 2, "matrix_scan: unknown mode");
+  SL_CHECK(mode >= 0 && mode <= 3, "matrix_scan: unknown mode");
   SL_CHECK(S >= 0 && T >= 0 && H > 0 && G > 0 && H % G == 0 && Dv > 0, "matrix_scan: sizes must be positive");
   SL_CHECK(D >= 1 && D <= 64 * SCAN_ROWS, "matrix_scan: at most 512 key channels a head");
   SL_CHECK(q_col >= 0 && k_col >= 0 && v_col >= 0 && q_col + G * D <= src_stride && k_col + G * D <= src_stride &&
            v_col + H * Dv <= src_stride, "matrix_scan: q, k or v do not fit the rows");
-  SL_CHECK(mode == SCAN_LSTM || log_decay != nullptr, "matrix_scan: decays are missing");
+  SL_CHECK(mode == SCAN_LSTM || mode == SCAN_SSD || log_decay != nullptr, "matrix_scan: decays are missing");
+  SL_CHECK(mode != SCAN_SSD || (rates != nullptr && step_bias != nullptr && skip != nullptr),
+           "matrix_scan: the state-space form needs rates, step biases and skips per head");
   SL_CHECK(mode == SCAN_DECAY || (gates != nullptr && i_col >= 0 && i_col + H <= gate_stride),
            "matrix_scan: gates are missing or do not fit their rows");
   SL_CHECK(mode != SCAN_LSTM || (f_col >= 0 && f_col + H <= gate_stride && cap > 0.f),
@@ -499,53 +516,64 @@ extern "C" const char* sl_matrix_scan(int mode, const float* src, int src_stride
   while (P * SCAN_ROWS < D) P <<= 1;
   const int cols = 256 / P, Dp = P * SCAN_ROWS;
   const int CH = min(min(16, 2048 / Dp), 8 * P);       // 8 values a thread of each kind a chunk
-  const size_t lds = 2 * (size_t)CH * ((mode == SCAN_LSTM ? 2 : 3) * Dp + 2 * cols + 4) * sizeof(float);   // two halves
+  const bool scalar = mode == SCAN_LSTM || mode == SCAN_SSD;
+  const size_t lds = 2 * (size_t)CH * ((scalar ? 2 : 3) * Dp + 2 * cols + 4) * sizeof(float);   // two halves
   const MatrixScan a{src, src_stride, q_col, k_col, v_col, H, G, D, Dv, log_decay, q_scale, gates, gate_stride,
-                     i_col, f_col, cap, state, state_stride, cu_q, positions, slots, write, out};
+                     i_col, f_col, rates, step_bias, skip, cap, state, state_stride, cu_q, positions, slots, write, out};
   const int vcols = mode == SCAN_LSTM ? cols - 1 : cols;       // (the matrix LSTM's last column group carries n)
   const dim3 grid(S, H, (Dv + vcols - 1) / vcols);
   if (mode == SCAN_DECAY) matrix_scan_kernel<SCAN_DECAY, SCAN_ROWS><<<grid, 512, lds, stream>>>(a, P, CH);
   else if (mode == SCAN_DELTA) matrix_scan_kernel<SCAN_DELTA, SCAN_ROWS><<<grid, 512, lds, stream>>>(a, P, CH);
+  else if (mode == SCAN_SSD) matrix_scan_kernel<SCAN_SSD, SCAN_ROWS><<<grid, 512, lds, stream>>>(a, P, CH);
   else matrix_scan_kernel<SCAN_LSTM, SCAN_ROWS><<<grid, 512, lds, stream>>>(a, P, CH);
   return sl_launch_status();
 }
 
 // ------------------------------------------------------------------ read-out: norm, gain, gate
 // One wavefront per (token, head): o / sqrt(mean(o^2) + eps) * w * act(gate); act 0: sigmoid, 1: silu.
+// gate_first: the gate comes before the norm, x = o * act(gate), then x / sqrt(mean(x^2) + eps) * w.
 __global__ __launch_bounds__(64) void head_norm_gate_kernel(const float* __restrict__ o, int H, int Dv,
                                                             const float* __restrict__ w, int per_head, float eps,
                                                             const float* __restrict__ gate, int gate_stride,
-                                                            int gate_col, int act, act_t* __restrict__ out) {
+                                                            int gate_col, int act, int gate_first,
+                                                            act_t* __restrict__ out) {
   const size_t t = blockIdx.x;
   const int h = blockIdx.y, lane = threadIdx.x;
   const float* x = o + (t * H + h) * Dv;
-  float ss = 0.f;
-  for (int d = lane; d < Dv; d += 64) ss += x[d] * x[d];
-  const float inv = 1.f / sqrtf(wave_sum(ss) / (float)Dv + eps);
   const float* gr = gate + t * gate_stride + gate_col + h * Dv;
   const float* wr = w + (per_head ? h * Dv : 0);
+  float ss = 0.f;
+  for (int d = lane; d < Dv; d += 64) {
+    float v = x[d];
+    if (gate_first) {
+      const float z = gr[d];
+      v *= act == 0 ? sigmoidf_(z) : z * sigmoidf_(z);
+    }
+    ss += v * v;
+  }
+  const float inv = 1.f / sqrtf(wave_sum(ss) / (float)Dv + eps);
   for (int d = lane; d < Dv; d += 64) {
     const float z = gr[d];
     const float gv = act == 0 ? sigmoidf_(z) : z * sigmoidf_(z);
-    out[(t * H + h) * Dv + d] = from_f<act_t>(x[d] * inv * wr[d] * gv);
+    out[(t * H + h) * Dv + d] = from_f<act_t>(gate_first ? (x[d] * gv) * inv * wr[d] : x[d] * inv * wr[d] * gv);
   }
 }
 
 extern "C" const char* sl_head_norm_gate(const float* o, int T, int H, int Dv, const float* w, int per_head,
                                          float eps, const float* gate, int gate_stride, int gate_col, int act,
-                                         void* out, hipStream_t stream) {
+                                         int gate_first, void* out, hipStream_t stream) {
   SL_CHECK(T >= 0 && H > 0 && Dv > 0, "head_norm_gate: sizes must be positive");
   SL_CHECK(gate_col >= 0 && gate_col + H * Dv <= gate_stride, "head_norm_gate: the gates do not fit their rows");
   SL_CHECK(act == 0 || act == 1, "head_norm_gate: the gate is sigmoid (0) or silu (1)");
   if (T == 0) return nullptr;
   head_norm_gate_kernel<<<dim3(T, H), 64, 0, stream>>>(o, H, Dv, w, per_head, eps, gate, gate_stride, gate_col,
-                                                       act, (act_t*)out);
+                                                       act, gate_first, (act_t*)out);
   return sl_launch_status();
 }
 
 // ------------------------------------------------------------------ softmax attention's q, k, v
 // buf row: q [H][D], k [G][D], v [G][Dv] (float).  q and k are divided by the root mean square of
-// all their heads together and multiplied by a gain of that size, then the first `rot` channels
+// all their heads together and multiplied by a gain of that size (no gains: no norm), then the first `rot` channels
 // of every head turn in halves (channel i with i + rot / 2, angle of cos/sin column i).  q leaves
 // in the activation type; k and v go to the token's place in the pages.  One block per token.
 __global__ void projnorm_rope_store_kernel(const float* __restrict__ buf, int stride, int H, int G, int D, int Dv,
@@ -558,10 +586,14 @@ __global__ void projnorm_rope_store_kernel(const float* __restrict__ buf, int st
   const float* row = buf + t * stride;
   const int nq = H * D, nk = G * D, nv = G * Dv;
   float sq = 0.f, sk = 0.f;
-  for (int e = threadIdx.x; e < nq; e += blockDim.x) sq += row[e] * row[e];
-  for (int e = threadIdx.x; e < nk; e += blockDim.x) sk += row[nq + e] * row[nq + e];
-  const float iq = 1.f / sqrtf(block_sum(sq, scratch) / (float)nq + eps);
-  const float ik = 1.f / sqrtf(block_sum(sk, scratch) / (float)nk + eps);
+  const bool normed = qw != nullptr;
+  float iq = 1.f, ik = 1.f;
+  if (normed) {
+    for (int e = threadIdx.x; e < nq; e += blockDim.x) sq += row[e] * row[e];
+    for (int e = threadIdx.x; e < nk; e += blockDim.x) sk += row[nq + e] * row[nq + e];
+    iq = 1.f / sqrtf(block_sum(sq, scratch) / (float)nq + eps);
+    ik = 1.f / sqrtf(block_sum(sk, scratch) / (float)nk + eps);
+  }
   const int half = rot / 2;
   const float* cs = cosv != nullptr ? cosv + t * half : nullptr;
   const float* sn = sinv != nullptr ? sinv + t * half : nullptr;
@@ -574,11 +606,11 @@ __global__ void projnorm_rope_store_kernel(const float* __restrict__ buf, int st
     const float* w = is_q ? qw : kw;
     const float inv = is_q ? iq : ik;
     const int d = el % D;
-    float v = x[el] * inv * w[el];
+    float v = normed ? x[el] * inv * w[el] : x[el];
     if (d < rot) {
       const int i = d < half ? d : d - half;
       const int partner = d < half ? el + half : el - half;
-      const float o = x[partner] * inv * w[partner];
+      const float o = normed ? x[partner] * inv * w[partner] : x[partner];
       v = d < half ? v * cs[i] - o * sn[i] : v * cs[i] + o * sn[i];
     }
     if (is_q) q_out[t * nq + el] = from_f<act_t>(v);
@@ -597,6 +629,7 @@ extern "C" const char* sl_projnorm_rope_store(const float* buf, int stride, int 
   SL_CHECK((long long)(H + G) * D + (long long)G * Dv <= stride, "projnorm_rope_store: q, k and v do not fit the rows");
   SL_CHECK(rot >= 0 && rot % 2 == 0 && rot <= D, "projnorm_rope_store: the rotated width must be even and within a head");
   SL_CHECK(rot == 0 || (cosv != nullptr && sinv != nullptr), "projnorm_rope_store: cos and sin are missing");
+  SL_CHECK((qw == nullptr) == (kw == nullptr), "projnorm_rope_store: both gains or neither");
   SL_CHECK(slots == nullptr || (kc != nullptr && vc != nullptr), "projnorm_rope_store: pages are missing");
   if (T == 0) return nullptr;
   projnorm_rope_store_kernel<<<T, 256, 0, stream>>>(buf, stride, H, G, D, Dv, qw, kw, eps, rot, cosv, sinv, slots,

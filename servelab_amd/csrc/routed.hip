@@ -6,9 +6,10 @@
 //               expert's rows start, the list of row tiles (expert, first row, rows) that the
 //               grouped products walk, and each pair's place in the sorted order
 //   grouped     y[row] = W[expert of row] x[row]: one launch over all experts, a workgroup per
-//               (row tile, column tile); the gated form computes silu(gate) * up of an expert's
-//               stacked [gate; up] matrix
-//   combine     out[token] = base[token] + sum over its choices of share * y[place of the pair]
+//               (row tile, column tile); the gated form computes act(gate) * up of an expert's
+//               stacked [gate; up] matrix, the activated form act(W x) of a single one
+//   combine     out[token] = g base[token] + sum over its choices of share * y[place of the pair],
+//               g = 1 or the sigmoid of one number per token
 //
 // No launch depends on the routing: the grids are sized for the worst case (pairs / tile rows
 // + experts tiles) and workgroups beyond the tiles in use leave at once, so a step is a fixed
@@ -136,8 +137,9 @@ struct Grouped {
   const int* tiles;          // [max_tiles][3]
   int sub;                   // row tiles hold 16 * sub rows
   int N, K;
-  act_t* out_act;            // gated: [rows][N]
+  act_t* out_act;            // gated and activated: [rows][N]
   float* out_f32;            // plain: [rows][N]
+  int act;                   // the activation (common.h); 0 with out_f32
   int max_tiles, col_blocks; // the matrix-core kernels' launch: max_tiles x col_blocks workgroups in a row
 };
 
@@ -158,7 +160,7 @@ __device__ __forceinline__ bool grouped_place(const Grouped& a, int& tile, int& 
 // 256 threads: thread (row = tid / 16, lane16 = tid % 16) owns columns lane16 + 16 u, u < 4, of a
 // 16 x 64 tile.  x and W go through LDS in chunks of 32 values of k; sums are float.
 template <bool GATED>
-__global__ __launch_bounds__(256) void grouped_product_kernel(const Grouped a) {
+__global__ __launch_bounds__(256) void grouped_product_kernel(const Grouped a) {   // (not GATED: plain or activated)
   const int* tl = a.tiles + 3 * (blockIdx.x / a.sub);
   const int part = blockIdx.x % a.sub;                  // which 16 rows of the row tile
   const int rows = min(RT_ROWS, tl[2] - RT_ROWS * part);
@@ -206,12 +208,9 @@ __global__ __launch_bounds__(256) void grouped_product_kernel(const Grouped a) {
     const int n = n0 + l + 16 * u;
     if (n >= a.N) continue;
     const size_t at = (size_t)(row0 + r) * a.N + n;
-    if (GATED) {
-      const float g = acc[u];
-      a.out_act[at] = from_f<act_t>(g / (1.f + expf(-g)) * acc2[u]);
-    } else {
-      a.out_f32[at] = acc[u];
-    }
+    if (GATED) a.out_act[at] = from_f<act_t>(sl_act(acc[u], a.act) * acc2[u]);
+    else if (a.act) a.out_act[at] = from_f<act_t>(sl_act(acc[u], a.act));
+    else a.out_f32[at] = acc[u];
   }
 }
 
@@ -293,10 +292,12 @@ __global__ __launch_bounds__(64 * WR * WC) void grouped_product_mfma_kernel(cons
       if (GATED) {
         rt_bf16x4 r;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const float g = acc[v][u][c];
-          r[c] = (__bf16)(g / (1.f + expf(-g)) * acc2[v][u][c]);
-        }
+        for (int c = 0; c < 4; ++c) r[c] = (__bf16)(sl_act(acc[v][u][c], a.act) * acc2[v][u][c]);
+        *(rt_bf16x4*)(a.out_act + at + 16 * u) = r;
+      } else if (a.act) {
+        rt_bf16x4 r;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) r[c] = (__bf16)sl_act(acc[v][u][c], a.act);
         *(rt_bf16x4*)(a.out_act + at + 16 * u) = r;
       } else {
         *(rt_f32x4*)(a.out_f32 + at + 16 * u) = acc[v][u];
@@ -407,10 +408,12 @@ __global__ __launch_bounds__(256, 2) void grouped_product_staged_kernel(const Gr
       if (GATED) {
         rt_bf16x4 r;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const float g = acc[v][u][c];
-          r[c] = (__bf16)(g / (1.f + expf(-g)) * acc[v][NU + u][c]);
-        }
+        for (int c = 0; c < 4; ++c) r[c] = (__bf16)(sl_act(acc[v][u][c], a.act) * acc[v][NU + u][c]);
+        *(rt_bf16x4*)(a.out_act + at + 16 * u) = r;
+      } else if (a.act) {
+        rt_bf16x4 r;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) r[c] = (__bf16)sl_act(acc[v][u][c], a.act);
         *(rt_bf16x4*)(a.out_act + at + 16 * u) = r;
       } else {
         *(rt_f32x4*)(a.out_f32 + at + 16 * u) = acc[v][u];
@@ -422,12 +425,15 @@ __global__ __launch_bounds__(256, 2) void grouped_product_staged_kernel(const Gr
 
 extern "C" const char* sl_grouped_product(const void* x, const int* order, int top, const void* w, const int* tiles,
                                           int w_tiled, int max_tiles, int tile_rows, int N, int K, int gated,
-                                          void* out, hipStream_t stream) {
+                                          int act, void* out, hipStream_t stream) {
+  // gated: act(gate) * up into the activation type; else act != 0: act(W x) into the activation type;
+  // else plain float sums
   SL_CHECK(max_tiles >= 0 && N > 0 && K > 0 && top >= 1, "grouped_product: sizes must be positive");
+  SL_CHECK(act >= 0 && act <= SL_ACT_RELU2 && (!gated || act), "grouped_product: unknown activation, or a gate without one");
   SL_CHECK(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "grouped_product: row tiles hold 16, 64 or 128 rows");
   if (max_tiles == 0) return nullptr;
   Grouped a{(const act_t*)x, order, top, (const act_t*)w, w_tiled, tiles, tile_rows / RT_ROWS, N, K,
-            gated ? (act_t*)out : nullptr, gated ? nullptr : (float*)out, max_tiles, 1};
+            act ? (act_t*)out : nullptr, act ? nullptr : (float*)out, act, max_tiles, 1};
 #if !defined(SL_F32)
   if (K % 32 == 0 && N % 16 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0) {
     // (a one-dimensional launch of max_tiles x col_blocks workgroups, rounded up to the eight dies)
@@ -459,12 +465,14 @@ extern "C" const char* sl_grouped_product(const void* x, const int* order, int t
 }
 
 // ------------------------------------------------------------------ combine
-// out[t] = base[t] + sum_k shares[t][k] * y[place_of[t top + k]], float sums, choices in their order.
+// out[t] = g[t] base[t] + sum_k shares[t][k] * y[place_of[t top + k]], float sums, choices in their order;
+// g[t] = sigmoid(base_gate[t * gate_stride]) when base_gate is given, else 1.
 __global__ __launch_bounds__(256) void routed_combine_kernel(const float* __restrict__ y,
                                                              const int* __restrict__ place_of,
                                                              const float* __restrict__ shares, int top,
-                                                             const act_t* __restrict__ base, int H,
-                                                             act_t* __restrict__ out) {
+                                                             const act_t* __restrict__ base,
+                                                             const float* __restrict__ base_gate, int gate_stride,
+                                                             int H, act_t* __restrict__ out) {
   __shared__ int place[64];
   __shared__ float share[64];
   const size_t t = blockIdx.x;
@@ -476,15 +484,17 @@ __global__ __launch_bounds__(256) void routed_combine_kernel(const float* __rest
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= H) return;
   float v = base != nullptr ? to_f(base[t * H + c]) : 0.f;
+  if (base_gate != nullptr) v *= 1.f / (1.f + expf(-base_gate[t * gate_stride]));
   for (int k = 0; k < top; ++k) v += share[k] * y[(size_t)place[k] * H + c];
   out[t * H + c] = from_f<act_t>(v);
 }
 
 extern "C" const char* sl_routed_combine(const float* y, const int* place_of, const float* shares, int T, int top,
-                                         const void* base, int H, void* out, hipStream_t stream) {
+                                         const void* base, const float* base_gate, int gate_stride, int H,
+                                         void* out, hipStream_t stream) {
   SL_CHECK(T >= 0 && top >= 1 && top <= 64 && H > 0, "routed_combine: sizes must be positive, at most 64 choices");
   if (T == 0) return nullptr;
-  routed_combine_kernel<<<dim3(T, (H + 255) / 256), 256, 0, stream>>>(y, place_of, shares, top, (const act_t*)base, H,
-                                                                    (act_t*)out);
+  routed_combine_kernel<<<dim3(T, (H + 255) / 256), 256, 0, stream>>>(y, place_of, shares, top, (const act_t*)base,
+                                                                    base_gate, gate_stride, H, (act_t*)out);
   return sl_launch_status();
 }

@@ -320,7 +320,8 @@ extern "C" const char* sl_headnorm_store(void* buf, int stride, int T, int nh, i
 }
 
 // ---------------------------------------------------------------------------
-// A latent row and its rotated part.  buf row t holds, from column down_off on,
+// A latent row and its rotated part.  The query heads of token t lie in qbuf row t
+// and, in dbuf row t (which may be the same rows) from column down_off on,
 // [C channels | R channels]: the first C are divided by their root mean square
 // and multiplied by a gain, and are the latent; of the last R the first `rot`
 // are rotated by the token's angles (pair i, i + rot / 2), the rest pass.  Both
@@ -330,12 +331,12 @@ extern "C" const char* sl_headnorm_store(void* buf, int stride, int T, int nh, i
 // One wavefront per (token, unit): unit 0 the latent row, unit 1 + h head h.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(64) void latent_store_kernel(
-    const act_t* __restrict__ buf, int stride, int nh, int D, int R, int C, int down_off, int rot,
-    const float* __restrict__ gain, float eps, const float* __restrict__ cosv,
+    const act_t* __restrict__ qbuf, int q_stride, const act_t* __restrict__ dbuf, int stride, int nh, int D, int R,
+    int C, int down_off, int rot, const float* __restrict__ gain, float eps, const float* __restrict__ cosv,
     const float* __restrict__ sinv, const int* __restrict__ slots, act_t* __restrict__ kc, int page,
     act_t* __restrict__ q_out) {
   const int t = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
-  const act_t* row = buf + (size_t)t * stride;
+  const act_t* row = dbuf + (size_t)t * stride;
   const int half = rot / 2;
   const act_t* src;
   act_t* dst;
@@ -356,7 +357,7 @@ __global__ __launch_bounds__(64) void latent_store_kernel(
     dst = krow + C;
   } else {
     const int h = unit - 1;
-    src = row + (size_t)h * (D + R) + D;
+    src = qbuf + (size_t)t * q_stride + (size_t)h * (D + R) + D;
     dst = q_out + ((size_t)t * nh + h) * (C + R) + C;
   }
   for (int i = lane; i < half; i += 64) {
@@ -368,20 +369,49 @@ __global__ __launch_bounds__(64) void latent_store_kernel(
   for (int d = rot + lane; d < R; d += 64) dst[d] = src[d];
 }
 
-extern "C" const char* sl_latent_store(const void* buf, int stride, int T, int nh, int D, int R, int C,
+extern "C" const char* sl_latent_store(const void* qbuf, int q_stride, const void* buf, int stride, int T, int nh,
+                                       int D, int R, int C,
                                        int down_off, int rot, const float* gain, float eps,
                                        const float* cosv, const float* sinv, const int* slots, void* kc,
                                        int page, void* q_out, hipStream_t stream) {
   SL_CHECK(T >= 0 && nh > 0 && D > 0 && R > 0 && C > 0, "latent_store: sizes must be positive");
   SL_CHECK(rot % 2 == 0 && rot >= 0 && rot <= R, "latent_store: the rotated width must be even and within R");
-  SL_CHECK(down_off >= nh * (D + R) && stride >= down_off + C + R, "latent_store: rows are too short");
+  SL_CHECK(down_off >= 0 && stride >= down_off + C + R && q_stride >= nh * (D + R) &&
+           (qbuf != buf || down_off >= nh * (D + R)), "latent_store: rows are too short");
   SL_CHECK(nh + 1 <= 65535, "latent_store: too many heads");
   SL_CHECK(rot == 0 || (cosv != nullptr && sinv != nullptr), "latent_store: a rotation needs its tables");
   SL_CHECK(gain != nullptr && q_out != nullptr, "latent_store: gain and q_out are required");
   SL_CHECK(slots == nullptr || (kc != nullptr && page > 0), "latent_store: a cache write needs the pages");
   if (T == 0) return nullptr;
   latent_store_kernel<<<dim3(T, nh + 1), 64, 0, stream>>>(
-      (const act_t*)buf, stride, nh, D, R, C, down_off, rot, gain, eps, cosv, sinv, slots, (act_t*)kc,
-      page, (act_t*)q_out);
+      (const act_t*)qbuf, q_stride, (const act_t*)buf, stride, nh, D, R, C, down_off, rot, gain, eps, cosv, sinv,
+      slots, (act_t*)kc, page, (act_t*)q_out);
+  return sl_launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// The RMS norm of a slice of columns: out[t][c] = x[t][col + c] * rsqrt(mean_c x^2 + eps) * gain[c],
+// sums in float.  One wavefront per token (a latent has few channels).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void slice_rmsnorm_kernel(const act_t* __restrict__ buf, int stride, int col, int n,
+                                                           const float* __restrict__ gain, float eps,
+                                                           act_t* __restrict__ out) {
+  const size_t t = blockIdx.x;
+  const act_t* x = buf + t * stride + col;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < n; d += 64) {
+    const float v = to_f(x[d]);
+    ss += v * v;
+  }
+  const float inv = 1.f / sqrtf(wave_sum(ss) / (float)n + eps);
+  for (int d = threadIdx.x; d < n; d += 64) out[t * n + d] = from_f<act_t>(to_f(x[d]) * inv * gain[d]);
+}
+
+extern "C" const char* sl_slice_rmsnorm(const void* buf, int stride, int col, int n, const float* gain, float eps,
+                                        int T, void* out, hipStream_t stream) {
+  SL_CHECK(T >= 0 && n > 0 && col >= 0 && col + n <= stride, "slice_rmsnorm: the slice does not fit the rows");
+  SL_CHECK(gain != nullptr, "slice_rmsnorm: the gain is required");
+  if (T == 0) return nullptr;
+  slice_rmsnorm_kernel<<<T, 64, 0, stream>>>((const act_t*)buf, stride, col, n, gain, eps, (act_t*)out);
   return sl_launch_status();
 }

@@ -1,8 +1,11 @@
 """Embedding gather, residual add + RMSNorm (with the products the norm runs or adds up itself),
-and the silu-multiply of a gate/up product."""
+the activation of a gate times its up product, and plain activations."""
+import ctypes
+
 import torch
 
-from .values import Deferred, KernelError, PartialSums, ScaledRows, TiledRows, _c_float, _p
+from .values import (Deferred, KernelError, PartialSums, ScaledRows, TiledRows, _c_float, _p,
+                     activation_code)
 
 
 class NormOps:
@@ -105,6 +108,12 @@ class NormOps:
         return ScaledRows(out, parts, eps, tiled=tiled)
 
     def silu_mul(self, gate_up, block=None):
+        return self.gate_mul(gate_up, block, "silu")
+
+    def gate_mul(self, gate_up, block=None, activation="silu"):
+        """act(gate) * up of rows that hold gate and up interleaved in blocks of ``block`` columns
+        (default: halves); ``activation``: "silu" or "relu"."""
+        code = activation_code(activation, ("silu", "relu"))
         T, two_i = gate_up.shape
         if two_i % 2:
             raise KernelError("silu_mul: the row must hold gate and up of equal width")
@@ -114,5 +123,31 @@ class NormOps:
             raise KernelError(f"silu_mul: block {block} does not divide the width {inter}")
         self._check(gate_up, self.act_dtype, None, "gate_up")
         out = self._new((T, inter))
-        self._call("elementwise", "sl_silu_mul", _p(gate_up), _p(out), T, inter, block)
+        self._call("elementwise", "sl_gate_mul", _p(gate_up), _p(out), T, inter, block, code)
+        return out
+
+    def activate(self, x, activation):
+        """act(x) in place, in float; ``activation``: "silu", "relu" or "relu2" (relu squared)."""
+        self._check(x, self.act_dtype, None, "x")
+        self._call("elementwise", "sl_activate", _p(x), _p(x), ctypes.c_longlong(x.numel()),
+                   activation_code(activation))
+        return x
+
+    def add_normed_rmsnorm(self, resid, y, y_weight, y_eps, weight, eps, rows=None):
+        """A sublayer's output ``y`` joins the float32 stream through an RMS norm of its own, and the
+        norm of the sublayer that reads the stream next follows in the same kernel:
+        v = resid + y / sqrt(mean(y^2) + y_eps) * y_weight, returned v / sqrt(mean(v^2) + eps) * weight.
+        ``rows`` None: every row, and v goes back into ``resid``; else (int32) only those rows are
+        computed and returned, and the stream stays as it is."""
+        T, H = resid.shape
+        self._check(resid, torch.float32, None, "residual stream")
+        self._check(y, self.act_dtype, (T, H), "sublayer output")
+        self._check(y_weight, torch.float32, (H,), "output norm weight")
+        self._check(weight, torch.float32, (H,), "norm weight")
+        if rows is not None:
+            self._check(rows, torch.int32, (rows.shape[0],), "rows")
+        R = T if rows is None else rows.shape[0]
+        out = self._new((R, H))
+        self._call("norm", "sl_add_normed_rmsnorm", _p(resid), _p(y), _p(y_weight), _c_float(y_eps), _p(rows),
+                   _p(weight), _c_float(eps), _p(out), R, H)
         return out

@@ -11,12 +11,12 @@ from typing import NamedTuple
 
 import torch
 
-from .values import KernelError, _c_float, _p
+from .values import KernelError, _c_float, _p, activation_code
 
 _ll = ctypes.c_longlong
 
 _EXPAND_MODES = {"plain": 0, "log_sigmoid": 1, "rate_softplus": 2}
-_SCAN_DECAY, _SCAN_DELTA, _SCAN_LSTM = 0, 1, 2
+_SCAN_DECAY, _SCAN_DELTA, _SCAN_LSTM, _SCAN_SSD = 0, 1, 2, 3
 _TILE_ROWS = (16, 64, 128)    # rows of a row tile of the grouped products (routed.hip)
 
 
@@ -112,9 +112,9 @@ class RecurrentOps:
         return out
 
     def short_conv(self, buf, col, taps, state, state_off, batch, write, unit_heads=0, unit_dim=0,
-                   unit_eps=1e-6, scaled_heads=0, scale=1.0):
+                   unit_eps=1e-6, scaled_heads=0, scale=1.0, bias=None):
         """silu of a causal convolution over time per channel of buf[:, col:col + C] (``taps``
-        [C, n], the last one the token's own).  The n - 1 inputs before a step come from the
+        [C, n], the last one the token's own; ``bias`` [C] is added before the silu).  The n - 1 inputs before a step come from the
         sequence's state slot at ``state_off`` ([n - 1, C], zeros at a sequence's start), and the
         step's last n - 1 inputs go back there.  The first ``unit_heads`` heads of ``unit_dim``
         channels are divided by sqrt(sum x^2 + unit_eps), the first ``scaled_heads`` of them also
@@ -122,17 +122,19 @@ class RecurrentOps:
         T, stride = self._f32_rows(buf, "projected rows")
         C, n = taps.shape
         self._check(taps, torch.float32, None, "taps")
+        if bias is not None:
+            self._check(bias, torch.float32, (C,), "convolution bias")
         self._sequences(batch, T)
         slot_size = self._state(state, state_off + (n - 1) * C)
         out = self._new((T, C), torch.float32)
-        self._call(self._lazy("recurrent"), "sl_short_conv", _p(buf), stride, col, C, n, _p(taps), _p(state),
+        self._call(self._lazy("recurrent"), "sl_short_conv", _p(buf), stride, col, C, n, _p(taps), _p(bias), _p(state),
                    _ll(slot_size), state_off, _p(batch.cu_q), _p(batch.positions), _p(batch.tok_seq),
                    _p(batch.state_slots), batch.num_seqs, T, int(bool(write)), unit_heads, unit_dim,
                    _c_float(unit_eps), scaled_heads, _c_float(scale), _p(out))
         return out
 
     def _scan(self, mode, src, q_col, k_col, v_col, H, G, D, Dv, log_decay, q_scale, gates, i_col, f_col,
-              cap, state, batch, write):
+              cap, state, batch, write, rates=None, step_bias=None, skip=None):
         T, stride = self._f32_rows(src, "q, k, v rows")
         self._sequences(batch, T)
         need = H * Dv * D + (H * D + H if mode == _SCAN_LSTM else 0)
@@ -147,7 +149,7 @@ class RecurrentOps:
         out = self._new((T, H * Dv), torch.float32)
         self._call(self._lazy("recurrent"), "sl_matrix_scan", mode, _p(src), stride, q_col, k_col, v_col, H, G,
                    D, Dv, _p(log_decay), _c_float(q_scale), _p(gates), gate_stride, i_col, f_col, _c_float(cap),
-                   _p(state), _ll(slot_size), _p(batch.cu_q), _p(batch.positions), _p(batch.state_slots),
+                   _p(rates), _p(step_bias), _p(skip), _p(state), _ll(slot_size), _p(batch.cu_q), _p(batch.positions), _p(batch.state_slots),
                    batch.num_seqs, T, int(bool(write)), _p(out))
         return out
 
@@ -171,10 +173,24 @@ class RecurrentOps:
         return self._scan(_SCAN_LSTM, buf, q_col, k_col, v_col, H, H, D, Dv, None, q_scale, buf, i_col, f_col,
                           cap, state, batch, write)
 
-    def head_norm_gate(self, o, H, Dv, weight, per_head, eps, gate, gate_col, activation):
+    def ssd_scan(self, src, x_col, b_col, c_col, H, G, N, P, steps, step_col, rates, step_bias, skip,
+                 state, batch, write):
+        """The state-space recurrence with one decay per head: with dt = softplus(steps[:, step_col + h]
+        + step_bias[h]), S' = exp(-exp(rates[h]) dt) S + dt B x^T and y = S'^T C + skip[h] x, where x
+        [H, P] lies at column ``x_col`` of ``src`` (float32 rows) and B and C, [G, N] each, at ``b_col``
+        and ``c_col`` (head h reads group h // (H / G)).  The slot holds S as [H, P, N] from 0 on; a
+        sequence whose first token is in the step starts from zero.  Returns float32 [T, H P]."""
+        for name, v in (("rates", rates), ("step biases", step_bias), ("skips", skip)):
+            self._check(v, torch.float32, (H,), name)
+        return self._scan(_SCAN_SSD, src, c_col, b_col, x_col, H, G, N, P, None, 1.0, steps, step_col, 0, 1.0,
+                          state, batch, write, rates=rates, step_bias=step_bias, skip=skip)
+
+    def head_norm_gate(self, o, H, Dv, weight, per_head, eps, gate, gate_col, activation, gate_first=False):
         """Each head of ``o`` [T, H Dv] (float32) divided by its root mean square, times ``weight``
         ([H Dv] when ``per_head``, else [Dv] for every head), times sigmoid or silu of
-        gate[:, gate_col + h Dv + d] (float32 rows).  Returns rows in the activation dtype."""
+        gate[:, gate_col + h Dv + d] (float32 rows).  ``gate_first``: the gate is applied before the
+        norm (a "head" is then any equal part of the row that is normed by itself).  Returns rows in
+        the activation dtype."""
         T, width = self._f32_rows(o, "read-out")
         if width != H * Dv:
             raise KernelError("head_norm_gate: the read-out is not [T, heads * channels]")
@@ -184,19 +200,23 @@ class RecurrentOps:
             raise KernelError("head_norm_gate: gates for another number of tokens, or an unknown activation")
         out = self._new((T, H * Dv))
         self._call(self._lazy("recurrent"), "sl_head_norm_gate", _p(o), T, H, Dv, _p(weight), int(bool(per_head)),
-                   _c_float(eps), _p(gate), gate_stride, gate_col, 0 if activation == "sigmoid" else 1, _p(out))
+                   _c_float(eps), _p(gate), gate_stride, gate_col, 0 if activation == "sigmoid" else 1,
+                   int(bool(gate_first)), _p(out))
         return out
 
     # ------------------------------- attention: norm over the projection, rotation, pages
     def projnorm_rope_store(self, buf, H, G, D, Dv, q_gain, k_gain, eps, rot, tables, slots, k_cache, v_cache,
                             page_size):
         """``buf`` (float32) holds q [H D], k [G D] and v [G Dv] side by side.  q and k are
-        RMS-normed over all their heads at once (gains of that size), the first ``rot`` channels of
+        RMS-normed over all their heads at once (gains of that size; both None: no norm), the first ``rot`` channels of
         every head rotated in halves by ``tables``; k and v go to the token's place in the pages
         (``slots`` None: no write); q comes back as [T, H D] in the activation dtype."""
         T, stride = self._f32_rows(buf, "projected rows")
-        self._check(q_gain, torch.float32, (H * D,), "q gain")
-        self._check(k_gain, torch.float32, (G * D,), "k gain")
+        if (q_gain is None) != (k_gain is None):
+            raise KernelError("projnorm_rope_store: both gains or neither")
+        if q_gain is not None:
+            self._check(q_gain, torch.float32, (H * D,), "q gain")
+            self._check(k_gain, torch.float32, (G * D,), "k gain")
         cos = sin = None
         if rot:
             cos, sin = tables.cos, tables.sin
@@ -248,20 +268,24 @@ class RecurrentOps:
             self._call("gemm", "sl_tile_weight", _p(w[e]), _p(tiled[e]), N, K, 16)
         return ExpertMatrices(tiled, w.shape, True)
 
-    def routed_experts(self, x, routing, w_gate_up, w_down, base=None):
-        """sum over a token's choices of share * down_e(silu(gate_e x) * up_e x), plus ``base``;
+    def routed_experts(self, x, routing, w_gate_up, w_down, base=None, activation="silu", gated=True,
+                       base_gate=None, base_gate_col=0):
+        """sum over a token's choices of share * down_e(act(gate_e x) * up_e x), plus ``base``;
         ``w_gate_up`` [E, 2 ff, width] holds an expert's gate rows before its up rows, ``w_down``
-        [E, width, ff].  Sums are float32; what lies between the two products is rounded to the
-        activation dtype."""
+        [E, width, ff].  ``gated`` False: an expert is down_e(act(up_e x)) and ``w_gate_up`` is
+        [E, ff, width].  ``base_gate`` (float32 rows): ``base`` is multiplied by the sigmoid of
+        base_gate[t, base_gate_col].  Sums are float32; what lies between the two products is
+        rounded to the activation dtype."""
+        code = activation_code(activation)
         if not isinstance(w_gate_up, ExpertMatrices):
             w_gate_up = ExpertMatrices(w_gate_up, w_gate_up.shape, False)
         if not isinstance(w_down, ExpertMatrices):
             w_down = ExpertMatrices(w_down, w_down.shape, False)
         T, K = x.shape
         E, two_ff, K2 = w_gate_up.shape
-        ff = two_ff // 2
+        ff = two_ff // 2 if gated else two_ff
         self._check(x, self.act_dtype, None, "x")
-        if w_gate_up.shape != (E, 2 * ff, K) or w_down.shape != (E, K, ff):
+        if w_gate_up.shape != (E, two_ff, K) or (gated and two_ff % 2) or w_down.shape != (E, K, ff):
             raise KernelError(f"routed_experts: matrices of {list(w_gate_up.shape)} and {list(w_down.shape)} "
                               f"for rows of {K} values")
         for m in (w_gate_up, w_down):
@@ -275,14 +299,23 @@ class RecurrentOps:
             raise KernelError("routed_experts: the routing is for another step or other experts")
         if base is not None:
             self._check(base, self.act_dtype, (T, K), "base")
+        gate_stride = 0
+        if base_gate is not None:
+            gate_stride = self._f32_rows(base_gate, "base gate")[1]
+            if base is None or base_gate.shape[0] != T or not 0 <= base_gate_col < gate_stride:
+                raise KernelError("routed_experts: the base's gate does not fit its rows, or there is no base")
         lib = self._lazy("routed")
         mid = self._new((n, ff))
         self._call(lib, "sl_grouped_product", _p(x), _p(routing.order), top, _p(w_gate_up.data),
-                   _p(routing.tiles), int(w_gate_up.tiled), max_tiles, routing.tile_rows, ff, K, 1, _p(mid))
+                   _p(routing.tiles), int(w_gate_up.tiled), max_tiles, routing.tile_rows, ff, K, int(bool(gated)), code,
+                   _p(mid))
         y = self._new((n, K), torch.float32)
         self._call(lib, "sl_grouped_product", _p(mid), None, 1, _p(w_down.data), _p(routing.tiles),
-                   int(w_down.tiled), max_tiles, routing.tile_rows, K, ff, 0, _p(y))
+                   int(w_down.tiled), max_tiles, routing.tile_rows, K, ff, 0, 0, _p(y))
         out = self._new((T, K))
-        self._call(lib, "sl_routed_combine", _p(y), _p(routing.place_of), _p(routing.shares), T, top, _p(base), K,
-                   _p(out))
+        gate_at = None
+        if base_gate is not None:
+            gate_at = ctypes.c_void_p(base_gate.data_ptr() + 4 * base_gate_col)
+        self._call(lib, "sl_routed_combine", _p(y), _p(routing.place_of), _p(routing.shares), T, top, _p(base),
+                   gate_at, gate_stride, K, _p(out))
         return out

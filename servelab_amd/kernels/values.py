@@ -114,3 +114,13 @@ class ScaledRows:
             return self.x
         T, K = self.x.shape
         return self.x.reshape(K // 32, T, 32).permute(1, 0, 2).reshape(T, K)
+
+
+# Activations as the kernels number them (csrc/common.h).
+ACTIVATIONS = {"silu": 1, "relu": 2, "relu2": 3}
+
+
+def activation_code(name, allowed=None) -> int:
+    if name not in ACTIVATIONS or (allowed is not None and name not in allowed):
+        raise KernelError(f"activation {name!r} is not one of {sorted(allowed or ACTIVATIONS)}")
+    return ACTIVATIONS[name]

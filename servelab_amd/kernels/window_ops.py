@@ -138,15 +138,33 @@ class WindowOps:
                    _p(k_cache) if slots is not None else None, _p(v_cache) if slots is not None else None,
                    page_size)
 
+    def slice_rmsnorm(self, buf, col, n, gain, eps):
+        """The RMS norm of columns col .. col + n of every row, times ``gain`` [n], in float32;
+        returns [T, n] in the activation dtype."""
+        T, stride = buf.shape
+        self._check(buf, self.act_dtype, None, "rows")
+        self._check(gain, torch.float32, (n,), "gain")
+        if col < 0 or col + n > stride:
+            raise KernelError("slice_rmsnorm: the slice does not fit the rows")
+        out = self._new((T, n))
+        self._call(self._lazy("window_attention"), "sl_slice_rmsnorm", _p(buf), stride, col, n, _p(gain),
+                   _c_float(eps), T, _p(out))
+        return out
+
     def latent_store(self, buf, nh, D, R, C, down_off, rot, gain, eps, tables, slots, k_cache,
-                     page_size, q_out):
-        """``buf`` [T, width] holds nh query heads of D + R channels and, from column ``down_off``,
+                     page_size, q_out, q_rows=None):
+        """``buf`` [T, width] holds nh query heads of D + R channels (``q_rows`` given: those rows
+        hold them instead, from column 0) and, from column ``down_off``,
         C + R channels: the first C, RMS-normed with ``gain``, and the last R with their first
         ``rot`` channels rotated by ``tables`` (cos and sin [T, rot / 2]) go to the token's key row
         (``slots`` None: no write); the last R channels of every query head are rotated the same
         way into ``q_out`` [T, nh, C + R] at channel C."""
         T, stride = buf.shape
         self._check(buf, self.act_dtype, None, "projected rows")
+        q_rows = buf if q_rows is None else q_rows
+        self._check(q_rows, self.act_dtype, None, "query rows")
+        if q_rows.dim() != 2 or q_rows.shape[0] != T or q_rows.shape[1] < nh * (D + R):
+            raise KernelError("latent_store: the query rows do not hold the heads")
         self._check(gain, torch.float32, (C,), "latent gain")
         self._check(q_out, self.act_dtype, (T, nh * (C + R)), "q in the latent's space")
         cos = sin = None
@@ -158,7 +176,8 @@ class WindowOps:
             self._check(k_cache, self.act_dtype, (k_cache.shape[0], 1, page_size, C + R), "latent pages")
             self._check(slots, torch.int32, (T,), "slots")
         lib = self._lazy("window_attention")
-        self._call(lib, "sl_latent_store", _p(buf), stride, T, nh, D, R, C, down_off, rot, _p(gain),
+        self._call(lib, "sl_latent_store", _p(q_rows), q_rows.shape[1], _p(buf), stride, T, nh, D, R, C, down_off,
+                   rot, _p(gain),
                    _c_float(eps), _p(cos), _p(sin), _p(slots), _p(k_cache) if slots is not None else None,
                    page_size, _p(q_out))
 

@@ -99,14 +99,16 @@ class ProjectionNormAttention(Mixer):
     (all heads of a token at once, a gain of that size) before the rotation, with biases on q,
     k, v and the output, keys of ``key_dim`` and values of ``value_dim`` channels, a score
     scale given from outside and float32 softmax weights.  The position encoding turns the
-    leading channels of a head in halves.  Causal; ``window`` None keeps every key."""
+    leading channels of a head in halves.  Causal; ``window`` None keeps every key.
+    ``projection_norm`` False: q and k go to the rotation as the projection left them (no gains
+    in the checkpoint); ``bias`` False: no biases."""
     graph_safe = True
 
     NAMES = {"q": "q", "k": "k", "v": "v", "out": "o", "q_bias": "q.b", "k_bias": "k.b",
              "v_bias": "v.b", "out_bias": "o.b", "q_norm": "q.norm", "k_norm": "k.norm"}
 
     def __init__(self, hidden_size, num_heads, num_kv_heads, key_dim, value_dim, scale, position,
-                 norm_eps, bias=True, window=None, names=None):
+                 norm_eps, bias=True, window=None, names=None, projection_norm=True):
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         self.hidden_size = int(hidden_size)
@@ -115,6 +117,7 @@ class ProjectionNormAttention(Mixer):
         self.scale, self.norm_eps = float(scale), float(norm_eps)
         self.position = position
         self.bias = bool(bias)
+        self.projection_norm = bool(projection_norm)
         self.window = None if not window else int(window)
         self.names = dict(self.NAMES, **(names or {}))
 
@@ -122,8 +125,10 @@ class ProjectionNormAttention(Mixer):
         n, h = self.names, self.hidden_size
         H, G, D, Dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
         specs = {n["q"]: ParamSpec((H * D, h)), n["k"]: ParamSpec((G * D, h)), n["v"]: ParamSpec((G * Dv, h)),
-                 n["q_norm"]: ParamSpec((H * D,), init="gain"), n["k_norm"]: ParamSpec((G * D,), init="gain"),
                  n["out"]: ParamSpec((h, H * Dv))}
+        if self.projection_norm:
+            specs.update({n["q_norm"]: ParamSpec((H * D,), init="gain"),
+                          n["k_norm"]: ParamSpec((G * D,), init="gain")})
         if self.bias:
             specs.update({n["q_bias"]: ParamSpec((H * D,)), n["k_bias"]: ParamSpec((G * D,)),
                           n["v_bias"]: ParamSpec((G * Dv,)), n["out_bias"]: ParamSpec((h,))})
@@ -151,8 +156,8 @@ class ProjectionNormAttention(Mixer):
                            tensors(n["v_bias"]).float(), torch.zeros(extra, device=w.device)], 0)
             self.b_in = rt.vector(b)
             self.b_o = rt.vector(tensors(n["out_bias"]))
-        self.q_gain = rt.vector(tensors(n["q_norm"]))
-        self.k_gain = rt.vector(tensors(n["k_norm"]))
+        self.q_gain = rt.vector(tensors(n["q_norm"])) if self.projection_norm else None
+        self.k_gain = rt.vector(tensors(n["k_norm"])) if self.projection_norm else None
         self.w_o = rt.linear_weight(tensors(n["out"]), delta=True)
 
     def forward(self, x, batch, cache, shared):

@@ -8,6 +8,10 @@ delta for the next norm to add.
 ParallelBlock: with x = Norm(h), h += Mixer(x) + FeedForward(x): one norm, both
 sublayers read its output; the block returns both outputs as its pending delta
 (a tuple), which the next norm adds to the stream in float32.
+
+SandwichBlock: h += Norm1b(Mixer(Norm1(h))); h += Norm2b(FeedForward(Norm2(h))): a norm before and
+after each sublayer.  The norm on an output and the norm before the next sublayer are one kernel
+call, so a block returns its last output with the norm that is still to be applied to it.
 """
 from .base import Block, prefixed
 
@@ -151,3 +155,53 @@ class PostNormBlock(Block):
             x = self.norm2.forward_post(resid, ops.materialize(self.feedforward.forward(x)))
         shared["stream rows"] = x
         return None
+
+
+class SandwichBlock(Block):
+    """A norm before and a norm after each sublayer: h += Norm1b(Mixer(Norm1(h))), then
+    h += Norm2b(FeedForward(Norm2(h))), all four of them ``RMSNorm`` parts.  A sublayer's output
+    waits, with the norm it has to pass, for the norm that reads the stream next
+    (``RMSNorm.normed`` -> ``NormedDelta``), which adds it.  ``feedforward`` may be None (then
+    there are no second norms).  Blocks of this kind follow each other or a block that leaves a
+    plain delta."""
+
+    def __init__(self, norm1, mixer, norm1b, norm2, feedforward, norm2b,
+                 names=("norm1.", "mix.", "norm1b.", "norm2.", "mlp.", "norm2b.")):
+        self.norm1, self.mixer, self.norm1b = norm1, mixer, norm1b
+        self.norm2, self.feedforward, self.norm2b = norm2, feedforward, norm2b
+        self.names = tuple(names)
+
+    @property
+    def graph_safe(self):
+        return all(part.graph_safe for _, part in self._children())
+
+    def _children(self):
+        parts = [(self.names[0], self.norm1), (self.names[1], self.mixer), (self.names[2], self.norm1b)]
+        if self.feedforward is not None:
+            parts += [(self.names[3], self.norm2), (self.names[4], self.feedforward), (self.names[5], self.norm2b)]
+        return parts
+
+    def cache_specs(self):
+        spec = self.mixer.cache_spec()
+        return [] if spec is None else [spec]
+
+    def param_specs(self):
+        specs = {}
+        for prefix, part in self._children():
+            for name, spec in part.param_specs().items():
+                specs[prefix + name] = spec
+        return specs
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        for prefix, part in self._children():
+            part.load(prefixed(prefix, tensors), rt)
+
+    def forward(self, resid, delta, batch, caches, shared):
+        x = self.norm1.forward(resid, delta)
+        a = self.mixer.forward(x, batch, caches[0] if caches else None, shared)
+        pending = self.norm1b.normed(a)
+        if self.feedforward is None:
+            return pending
+        x2 = self.norm2.forward(resid, pending)
+        return self.norm2b.normed(self.feedforward.forward(x2))

@@ -1,4 +1,5 @@
-"""Gated feed-forward (SwiGLU): down(silu(gate(x)) * up(x)), no biases.
+"""Gated feed-forward: down(act(gate(x)) * up(x)), no biases, act = silu (SwiGLU) or relu; and the
+plain one, down(act(up(x))), act = silu, relu or the square of relu.
 
 Reference: servelab/parallel/tp_model.py:56-68 (two GEMMs, silu, multiply, one
 GEMM).  Here gate and up are one GEMM over a matrix that holds the rows of Wg
@@ -17,8 +18,9 @@ class GatedMLP(FeedForward):
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu",
                  names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
-        if activation != "silu":
+        if activation not in ("silu", "relu"):
             raise ValueError(f"GatedMLP: activation '{activation}' is not supported")
+        self.activation = activation
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
         self.names = tuple(names)          # checkpoint names of the gate, up and down matrices
@@ -43,4 +45,33 @@ class GatedMLP(FeedForward):
 
     def forward(self, x):
         ops = self.rt.ops
-        return ops.gated_mlp(x, self.w_gate_up, self.block, self.w_down, defer=True)
+        if self.activation == "silu":
+            return ops.gated_mlp(x, self.w_gate_up, self.block, self.w_down, defer=True)
+        return ops.gated_mlp(x, self.w_gate_up, self.block, self.w_down, defer=True, activation=self.activation)
+
+
+class PlainMLP(FeedForward):
+    """down(act(up(x))) without a gate and without biases; ``activation``: "silu", "relu" or
+    "relu2" (the square of relu).  ``names``: checkpoint names of the up and down matrices."""
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "relu",
+                 names=("up", "down")):
+        if activation not in ("silu", "relu", "relu2"):
+            raise ValueError(f"PlainMLP: activation '{activation}' is not supported")
+        self.activation = activation
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.names = tuple(names)
+
+    def param_specs(self):
+        h, i = self.hidden_size, self.intermediate_size
+        return {self.names[0]: ParamSpec((i, h)), self.names[1]: ParamSpec((h, i))}
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        self.w_up = rt.linear_weight(tensors(self.names[0]))
+        self.w_down = rt.linear_weight(tensors(self.names[1]), delta=True)
+
+    def forward(self, x):
+        ops = self.rt.ops
+        return ops.linear(ops.activate(ops.linear(x, self.w_up, None), self.activation), self.w_down, None)

@@ -8,26 +8,50 @@ every use (servelab/parallel/tp_model.py:131-133) is fused in.
 from .base import Norm, ParamSpec
 
 
+class NormedDelta:
+    """A sublayer's output that joins the stream through an RMS norm of its own:
+    stream += y / sqrt(mean(y^2) + eps) * weight.  A block hands it on as its pending delta, and
+    the RMS norm that reads the stream next does the add and its own norm in one kernel call."""
+    __slots__ = ("y", "weight", "eps")
+
+    def __init__(self, y, weight, eps):
+        self.y, self.weight, self.eps = y, weight, float(eps)
+
+
 class RMSNorm(Norm):
+    """``offset``: the stored weight w acts as the gain offset + w (1 for weights kept around
+    zero); the sum is taken once at load, in float32."""
     graph_safe = True
 
-    def __init__(self, size: int, eps: float, name: str = "weight"):
+    def __init__(self, size: int, eps: float, name: str = "weight", offset: float = 0.0):
         self.size = int(size)
         self.eps = float(eps)
         self.name = name
+        self.offset = float(offset)
 
     def param_specs(self):
-        return {self.name: ParamSpec((self.size,), init="gain")}
+        return {self.name: ParamSpec((self.size,), init="gain" if not self.offset else "normal")}
 
     def load(self, tensors, rt):
         self.rt = rt
         self.weight = rt.vector(tensors(self.name))
+        if self.offset:
+            self.weight = (self.weight + self.offset).contiguous()
 
     def forward(self, resid, delta, fuse=False):
+        if isinstance(delta, NormedDelta):
+            return self.rt.ops.add_normed_rmsnorm(resid, delta.y, delta.weight, delta.eps, self.weight, self.eps)
         return self.rt.ops.add_rmsnorm(resid, delta, self.weight, self.eps, fuse=fuse)
 
     def forward_rows(self, resid, delta, rows, fuse=False):
+        if isinstance(delta, NormedDelta):
+            return self.rt.ops.add_normed_rmsnorm(resid, delta.y, delta.weight, delta.eps, self.weight, self.eps,
+                                                  rows=rows)
         return self.rt.ops.rows_add_rmsnorm(resid, delta, rows, self.weight, self.eps, fuse=fuse)
+
+    def normed(self, y):
+        """``y`` as a delta that joins the stream through this norm."""
+        return NormedDelta(self.rt.ops.materialize(y), self.weight, self.eps)
 
 
 class LayerNorm(Norm):

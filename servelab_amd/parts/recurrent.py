@@ -1,6 +1,6 @@
 """Mixers whose memory is a matrix per head, carried from token to token in a state slot.
 
-All three keep, per head, S [dim, vdim] in float32 and read a token's output as S^T q:
+All of them keep, per head, S [dim, vdim] in float32 and read a token's output as S^T q:
 
 ``MatrixLSTM``: scalar gates per head with a running maximum m (m_0 = 0):
     i = cap tanh(i~ / cap), f = logsigmoid(cap tanh(f~ / cap)), m' = max(f + m, i),
@@ -18,6 +18,12 @@ read-out sees the token's own write); g = exp(-exp(A_log_h) softplus(a + dt_bias
 key channel, a from a low-rank projection; the gain is shared by the heads and the sigmoid
 output gate comes from a low-rank projection.  The convolution's last taps - 1 inputs are part
 of the state.
+
+``StateSpaceMixer``: one projection gives a gate z, the inputs x, B and C (B and C shared by the
+heads of a group) and a step size per head; x, B and C pass a short causal convolution with a bias
+and silu; dt = softplus(dt~ + dt_bias_h); S' = exp(-exp(A_log_h) dt) S + dt B x^T (one decay for
+the whole head), y = S'^T C + D_h x; y times silu(z), then RMS-normed in equal parts with a gain
+over the whole row.  The convolution's last taps - 1 inputs are part of the state.
 
 Gates, decays, unit norms, state and read-out are float32 in both activation types; the input
 projection (one product for everything a mixer projects from its input) returns float32 sums.
@@ -203,6 +209,66 @@ class GatedDeltaRule(_MatrixMemoryMixer):
                            buf, at["beta"], cache.state, batch, cache.write)
         gate = ops.lowrank_expand(buf, at["gate_in"], self.gate_out, None, "plain", heads=H)
         y = ops.head_norm_gate(o, H, Dv, self.gain, False, self.norm_eps, gate, 0, "sigmoid")
+        return ops.linear(y, self.w_o, None)
+
+
+class StateSpaceMixer(_MatrixMemoryMixer):
+    NAMES = {"in": "in", "conv": "conv", "conv_bias": "conv.b", "step_bias": "dt_bias", "rate": "A_log",
+             "skip": "D", "norm": "norm", "out": "o"}
+
+    def __init__(self, hidden_size, heads, vdim, state, groups, conv, norm_groups, norm_eps, names=None):
+        if heads % groups or (heads * vdim) % norm_groups:
+            raise ValueError("heads must be a multiple of groups, heads * vdim of norm_groups")
+        self.hidden_size, self.heads, self.vdim, self.state = int(hidden_size), int(heads), int(vdim), int(state)
+        self.groups, self.conv, self.norm_groups = int(groups), int(conv), int(norm_groups)
+        self.norm_eps = float(norm_eps)
+        self.names = dict(self.NAMES, **(names or {}))
+
+    @property
+    def inner(self):
+        return self.heads * self.vdim
+
+    @property
+    def channels(self):
+        """What passes the convolution: x, B and C."""
+        return self.inner + 2 * self.groups * self.state
+
+    def param_specs(self):
+        n, h, H = self.names, self.hidden_size, self.heads
+        return {n["in"]: ParamSpec((2 * self.inner + 2 * self.groups * self.state + H, h)),
+                n["conv"]: ParamSpec((self.channels, self.conv)), n["conv_bias"]: ParamSpec((self.channels,)),
+                n["step_bias"]: ParamSpec((H,)), n["rate"]: ParamSpec((H,)), n["skip"]: ParamSpec((H,)),
+                n["norm"]: ParamSpec((self.inner,), init="gain"), n["out"]: ParamSpec((h, self.inner))}
+
+    def cache_spec(self):
+        return StateSpec((self.inner * self.state + (self.conv - 1) * self.channels,), "float32")   # S, last inputs
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        n = self.names
+        w = tensors(n["in"])
+        # the projection's rows are [z | x | B | C | dt]
+        self._load_in([("z", w[:self.inner]), ("xbc", w[self.inner:self.inner + self.channels]),
+                       ("dt", w[self.inner + self.channels:])], rt)
+        self.taps = rt.vector(tensors(n["conv"]))
+        self.conv_bias = rt.vector(tensors(n["conv_bias"]))
+        self.step_bias = rt.vector(tensors(n["step_bias"]))
+        self.rate = rt.vector(tensors(n["rate"]))
+        self.skip = rt.vector(tensors(n["skip"]))
+        self.gain = rt.vector(tensors(n["norm"]))
+        self.w_o = rt.linear_weight(tensors(n["out"]), delta=True)
+
+    def forward(self, x, batch, cache, shared):
+        ops, at = self.rt.ops, self.at
+        H, P, N, G = self.heads, self.vdim, self.state, self.groups
+        buf = self._project(x)
+        xbc = ops.short_conv(buf, at["xbc"], self.taps, cache.state, self.inner * N, batch, cache.write,
+                             bias=self.conv_bias)
+        y = ops.ssd_scan(xbc, 0, self.inner, self.inner + G * N, H, G, N, P, buf, at["dt"], self.rate,
+                         self.step_bias, self.skip, cache.state, batch, cache.write)
+        # the gate comes before the norm, which takes the row in `norm_groups` equal parts
+        y = ops.head_norm_gate(y, self.norm_groups, self.inner // self.norm_groups, self.gain, True,
+                               self.norm_eps, buf, at["z"], "silu", gate_first=True)
         return ops.linear(y, self.w_o, None)
 
 

@@ -1,7 +1,9 @@
 """A feed-forward of routed experts: every token goes through the ``top`` experts with the
 largest router logits, weighted by the softmax over those logits only, plus an optional shared
-expert that every token takes.  An expert is the gated feed-forward down(silu(gate x) * up x)
-without biases.  Router logits are float32 sums.
+expert that every token takes.  An expert is the gated feed-forward down(act(gate x) * up x)
+without biases (``gated`` False: down(act(up x)), from two matrices).  Router logits are float32
+sums, with a bias when ``router_bias``.  ``shared_gate``: the shared expert's output is multiplied
+by the sigmoid of one number per token, a projection of the input by a [1, width] matrix.
 
 The experts' matrices are stacked at load ([experts, 2 ff, width] with an expert's gate rows
 before its up rows, and [experts, width, ff]); the kernel table sorts the step's (token,
@@ -11,34 +13,46 @@ is a fixed list of launches whatever the routing.
 import torch
 
 from .base import FeedForward, ParamSpec
-from .feedforward import GatedMLP
+from .feedforward import GatedMLP, PlainMLP
 
 
 class RoutedExperts(FeedForward):
     graph_safe = True
 
-    def __init__(self, hidden_size, experts, top, ff, shared_ff=0, names=None):
+    def __init__(self, hidden_size, experts, top, ff, shared_ff=0, names=None, activation="silu", gated=True,
+                 router_bias=False, shared_gate=False):
         if not 1 <= top <= experts:
             raise ValueError("top must be between 1 and the number of experts")
+        if activation not in (("silu", "relu") if gated else ("silu", "relu", "relu2")):
+            raise ValueError(f"RoutedExperts: activation '{activation}' is not supported")
         self.hidden_size, self.experts, self.top, self.ff = int(hidden_size), int(experts), int(top), int(ff)
-        self.names = dict({"router": "router", "expert": "e{}.", "shared": "shared.",
-                           "gate": "gate", "up": "up", "down": "down"}, **(names or {}))
+        self.activation, self.gated, self.router_bias = activation, bool(gated), bool(router_bias)
+        self.names = dict({"router": "router", "router_bias": "router.b", "expert": "e{}.", "shared": "shared.",
+                           "shared_gate": "shared.sg", "gate": "gate", "up": "up", "down": "down"}, **(names or {}))
         n = self.names
-        self.shared = GatedMLP(hidden_size, shared_ff, names=(n["gate"], n["up"], n["down"])) \
-            if shared_ff else None
+        self.shared = None
+        if shared_ff:
+            self.shared = GatedMLP(hidden_size, shared_ff, activation, names=(n["gate"], n["up"], n["down"])) \
+                if gated else PlainMLP(hidden_size, shared_ff, activation, names=(n["up"], n["down"]))
+        self.shared_gate = bool(shared_gate) and self.shared is not None
 
     def param_specs(self):
         n, h, f = self.names, self.hidden_size, self.ff
         specs = {}
         for e in range(self.experts):
             p = n["expert"].format(e)
-            specs[p + n["gate"]] = ParamSpec((f, h))
+            if self.gated:
+                specs[p + n["gate"]] = ParamSpec((f, h))
             specs[p + n["up"]] = ParamSpec((f, h))
             specs[p + n["down"]] = ParamSpec((h, f))
         specs[n["router"]] = ParamSpec((self.experts, h))
+        if self.router_bias:
+            specs[n["router_bias"]] = ParamSpec((self.experts,))
         if self.shared is not None:
             for name, spec in self.shared.param_specs().items():
                 specs[n["shared"] + name] = spec
+        if self.shared_gate:
+            specs[n["shared_gate"]] = ParamSpec((1, h))
         return specs
 
     def load(self, tensors, rt):
@@ -46,24 +60,36 @@ class RoutedExperts(FeedForward):
         self.rt = rt
         n = self.names
         router = tensors(n["router"])
+        if self.shared_gate:           # the shared expert's gate is one more row of the router's product
+            router = torch.cat([router, tensors(n["shared_gate"]).reshape(1, -1)], 0)
         extra = -router.shape[0] % 8
         if extra:
             router = torch.cat([router, router.new_zeros(extra, router.shape[1])], 0)
         self.w_router = rt.linear_weight(router)
+        self.b_router = None
+        if self.router_bias:
+            b = torch.zeros(router.shape[0], dtype=torch.float32, device=router.device)
+            b[:self.experts] = tensors(n["router_bias"]).float()
+            self.b_router = rt.vector(b)
         gate_up, down = [], []
         for e in range(self.experts):
             p = n["expert"].format(e)
-            gate_up.append(torch.cat([tensors(p + n["gate"]), tensors(p + n["up"])], 0))
+            up = tensors(p + n["up"])
+            gate_up.append(torch.cat([tensors(p + n["gate"]), up], 0) if self.gated else up)
             down.append(tensors(p + n["down"]))
         prepare = getattr(rt.ops, "prepare_expert_matrices", lambda w, gated=False: w)   # (the kernel table's layout)
-        self.w_gate_up = prepare(rt.matrix(torch.stack(gate_up)), gated=True)            # [E, 2 ff, width]
+        self.w_gate_up = prepare(rt.matrix(torch.stack(gate_up)), gated=self.gated)      # [E, 2 ff | ff, width]
         self.w_down = prepare(rt.matrix(torch.stack(down)))                 # [E, width, ff]
         if self.shared is not None:
             self.shared.load(prefixed(n["shared"], tensors), rt)
 
     def forward(self, x):
         ops = self.rt.ops
-        logits = ops.linear(x, self.w_router, None, out_f32=True)
+        logits = ops.linear(x, self.w_router, self.b_router, out_f32=True)
         routing = ops.route_tokens(logits, self.experts, self.top)
         base = ops.materialize(self.shared.forward(x)) if self.shared is not None else None
-        return ops.routed_experts(x, routing, self.w_gate_up, self.w_down, base)
+        if self.gated and self.activation == "silu" and not self.shared_gate:
+            return ops.routed_experts(x, routing, self.w_gate_up, self.w_down, base)
+        return ops.routed_experts(x, routing, self.w_gate_up, self.w_down, base, activation=self.activation,
+                                  gated=self.gated, base_gate=logits if self.shared_gate else None,
+                                  base_gate_col=self.experts)

@@ -19,7 +19,10 @@ plus one rotated key part shared by the heads; score = (q_h . k_h + q_h' . k')
 [c | k'] of one kv head, and the attention runs in the latent's space: the
 query becomes [Wuk_h^T q_h | q_h'], the weighted sum of the cached c comes back
 through Wuv_h (both are products with one small matrix per head), so neither
-keys nor values of the heads are ever formed for cached tokens.
+keys nor values of the heads are ever formed for cached tokens.  With ``q_rank`` the queries
+pass a latent of their own: q = Wuq RMSNorm(Wdq x), the norm with a gain of ``q_rank`` channels.
+The rotation may pair halves or neighbouring channels: the rows that make the rotated channels
+are put into the order of halves at load (a score does not depend on the order of its terms).
 
 Every constant is a constructor parameter; checkpoint names are a parameter
 too (``names``).
@@ -126,17 +129,26 @@ class GatedWindowAttention(Mixer):
 
 
 _LATENT_NAMES = {"q": "q", "down": "dkv", "down_norm": "dkv.norm", "up_k": "uk", "up_v": "uv",
-                 "gate": "g", "out": "o"}
+                 "gate": "g", "out": "o", "q_down": "dq", "q_down_norm": "dq.norm", "q_up": "uq"}
+
+
+def _halves_order(rot: int, width: int, pairing: str) -> torch.Tensor:
+    """The order that puts ``width`` channels whose first ``rot`` turn in ``pairing`` pairs into
+    the order in which they turn in halves."""
+    if pairing == "half":
+        return torch.arange(width)
+    return torch.cat([torch.arange(0, rot, 2), torch.arange(1, rot, 2), torch.arange(rot, width)])
 
 
 class LatentWindowAttention(Mixer):
     graph_safe = True
 
     def __init__(self, hidden_size, num_heads, head_dim, rot_dim, value_dim, rank, scale, window,
-                 position, norm_eps=1e-6, gate=True, names=None):
+                 position, norm_eps=1e-6, gate=True, names=None, q_rank=None):
         """``position``: the encoding of the ``rot_dim`` rotated channels (a
-        ``PositionEncoding`` whose layout rotates its leading channels in
-        halves)."""
+        ``PositionEncoding`` whose layout rotates leading channels of them).
+        ``q_rank``: the width of the queries' latent (None: q is one projection
+        of the input)."""
         self.hidden_size = int(hidden_size)
         self.num_heads = int(num_heads)
         self.head_dim, self.rot_dim = int(head_dim), int(rot_dim)
@@ -146,14 +158,21 @@ class LatentWindowAttention(Mixer):
         self.position = position
         self.norm_eps = float(norm_eps)
         self.gate = bool(gate)
+        self.q_rank = None if not q_rank else int(q_rank)
         self.names = dict(_LATENT_NAMES, **(names or {}))
 
     def param_specs(self):
         n, h = self.names, self.hidden_size
         H, D, R, Dv, C = self.num_heads, self.head_dim, self.rot_dim, self.value_dim, self.rank
-        specs = {n["q"]: ParamSpec((H * (D + R), h)), n["down"]: ParamSpec((C + R, h)),
+        specs = {n["down"]: ParamSpec((C + R, h)),
                  n["down_norm"]: ParamSpec((C,), init="gain"),
                  n["up_k"]: ParamSpec((H * D, C)), n["up_v"]: ParamSpec((H * Dv, C))}
+        if self.q_rank:
+            specs.update({n["q_down"]: ParamSpec((self.q_rank, h)),
+                          n["q_down_norm"]: ParamSpec((self.q_rank,), init="gain"),
+                          n["q_up"]: ParamSpec((H * (D + R), self.q_rank))})
+        else:
+            specs[n["q"]] = ParamSpec((H * (D + R), h))
         if self.gate:
             specs[n["gate"]] = ParamSpec((H, h))
         specs[n["out"]] = ParamSpec((h, H * Dv))
@@ -172,10 +191,24 @@ class LatentWindowAttention(Mixer):
         if layout is None:
             self.rot = 0
         else:
-            if layout.pairing != "half" or layout.rot_dim > self.rot_dim:
-                raise ValueError("the rotated part takes an encoding that turns its leading channels in halves")
+            if layout.pairing not in ("half", "interleaved") or layout.rot_dim > self.rot_dim:
+                raise ValueError("the rotated part takes an encoding that turns leading channels of it, in "
+                                 "halves or in neighbouring pairs")
             self.rot = int(layout.rot_dim)
-        rows = [tensors(n["q"]), tensors(n["down"])]
+        R = self.rot_dim
+        order = _halves_order(self.rot, R, "half" if layout is None else layout.pairing)
+        w_q = tensors(n["q_up"] if self.q_rank else n["q"])
+        by_head = w_q.reshape(H, D + R, w_q.shape[1])
+        w_q = torch.cat([by_head[:, :D], by_head[:, D:][:, order.to(w_q.device)]], 1).reshape(w_q.shape)
+        w_down = tensors(n["down"])
+        w_down = torch.cat([w_down[:C], w_down[C:][order.to(w_down.device)]], 0)
+        if self.q_rank:
+            # [q's latent; down; gate] in one product, the queries in a second one from the normed latent
+            rows = [tensors(n["q_down"]), w_down]
+            self.w_q = rt.linear_weight(w_q)
+            self.q_gain = rt.vector(tensors(n["q_down_norm"]))
+        else:
+            rows = [w_q, w_down]
         if self.gate:
             rows.append(tensors(n["gate"]))
         self.w_in = rt.linear_weight(_padded_rows(rows))          # [q; down; gate] in one product
@@ -190,14 +223,20 @@ class LatentWindowAttention(Mixer):
         H, D, R, Dv, C = self.num_heads, self.head_dim, self.rot_dim, self.value_dim, self.rank
         group = batch.groups[cache.group]
         buf = ops.linear(x, self.w_in, None)
-        down_col = H * (D + R)
+        if self.q_rank:
+            down_col = self.q_rank
+            q_rows = ops.linear(ops.slice_rmsnorm(buf, 0, self.q_rank, self.q_gain, self.norm_eps), self.w_q, None)
+        else:
+            down_col = H * (D + R)
+            q_rows = buf
         g_col = down_col + C + R
         T = buf.shape[0]
         q_lat = torch.empty((T, H * (C + R)), dtype=buf.dtype, device=buf.device)
         tables = self.position.tables(batch, shared) if self.rot else None
         ops.latent_store(buf, H, D, R, C, down_col, self.rot, self.gain, self.norm_eps, tables,
-                         group.slots if cache.write else None, cache.k, cache.page_size, q_lat)
-        ops.head_products(buf, 0, H, D + R, self.to_latent, y=q_lat, y_col=0, y_head=C + R)
+                         group.slots if cache.write else None, cache.k, cache.page_size, q_lat,
+                         q_rows=q_rows if self.q_rank else None)
+        ops.head_products(q_rows, 0, H, D + R, self.to_latent, y=q_lat, y_col=0, y_head=C + R)
         attn = ops.window_attention(q_lat, 0, H, 1, C + R, C, cache.k, None, cache.page_size,
                                     group.block_tables, batch, self.scale, self.window, 0, None, None,
                                     buf if self.gate else None, g_col)

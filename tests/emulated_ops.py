@@ -47,12 +47,35 @@ class EmulatedOps:
         return y if out_f32 else y.to(self.act_dtype)
 
     def silu_mul(self, gate_up, block=None):
+        return self.gate_mul(gate_up, block, "silu")
+
+    @staticmethod
+    def _act(z, activation):
+        if activation == "silu":
+            return z * torch.sigmoid(z)
+        return torch.relu(z) if activation == "relu" else torch.relu(z) ** 2
+
+    def gate_mul(self, gate_up, block=None, activation="silu"):
         """gate and up interleaved in blocks of ``block`` columns (default: halves)."""
         T, inter = gate_up.shape[0], gate_up.shape[1] // 2
         block = inter if block is None else block
         gu = _f(gate_up).view(T, inter // block, 2, block)
         g, u = gu[:, :, 0].reshape(T, inter), gu[:, :, 1].reshape(T, inter)
-        return (g * torch.sigmoid(g) * u).to(self.act_dtype)
+        return (self._act(g, activation) * u).to(self.act_dtype)
+
+    def activate(self, x, activation):
+        return x.copy_(self._act(_f(x), activation).to(x.dtype))
+
+    def add_normed_rmsnorm(self, resid, y, y_weight, y_eps, weight, eps, rows=None):
+        """v = resid + y / sqrt(mean(y^2) + y_eps) * y_weight; returns v / sqrt(mean(v^2) + eps) *
+        weight.  rows None: v goes back into resid; else only those rows, resid untouched."""
+        y = _f(y)
+        v = resid + y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + y_eps) * y_weight
+        if rows is None:
+            resid.copy_(v)
+        else:
+            v = v[rows.long()]
+        return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * weight).to(self.act_dtype)
 
     def attend_and_project(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
                            batch, scale, window, w_out, bias=None, defer=False):
@@ -60,11 +83,11 @@ class EmulatedOps:
                                     batch, scale, window)
         return self.linear(attn, w_out, bias, defer=defer)
 
-    def gated_mlp(self, x, w_gate_up, block, w_down, defer=False):
-        return self.linear(self.gated_linear(x, w_gate_up, block), w_down, None, defer=defer)
+    def gated_mlp(self, x, w_gate_up, block, w_down, defer=False, activation="silu"):
+        return self.linear(self.gated_linear(x, w_gate_up, block, activation), w_down, None, defer=defer)
 
-    def gated_linear(self, x, w, block):
-        return self.silu_mul(self.linear(x, w, None), block)
+    def gated_linear(self, x, w, block, activation="silu"):
+        return self.gate_mul(self.linear(x, w, None), block, activation)
 
     # ----------------------------------------------------------------- rope
     def rope_tables(self, positions, inv_freq):
@@ -206,7 +229,7 @@ class EmulatedOps:
         raise ValueError(mode)
 
     def short_conv(self, buf, col, taps, state, state_off, batch, write, unit_heads=0, unit_dim=0,
-                   unit_eps=1e-6, scaled_heads=0, scale=1.0):
+                   unit_eps=1e-6, scaled_heads=0, scale=1.0, bias=None):
         """silu of a causal convolution over time per channel of buf[:, col:col + C] (taps [C, n],
         the last tap is the token's own); the n - 1 inputs before a step's first token come from
         state[slot, state_off:] laid out [n - 1, C] (oldest first; zeros at a sequence's start) and
@@ -221,6 +244,8 @@ class EmulatedOps:
             past = torch.zeros(n - 1, C) if fresh else keep.clone()
             full = torch.cat([past, x[a:b]], 0)
             y = sum(full[j:j + b - a] * taps[:, j] for j in range(n))
+            if bias is not None:
+                y = y + bias
             out[a:b] = y * torch.sigmoid(y)
             if write and n > 1:
                 keep.copy_(full[full.shape[0] - (n - 1):])
@@ -291,17 +316,43 @@ class EmulatedOps:
                 row[nS + nn:nS + nn + H].copy_(m)
         return out.view(T, H * Dv)
 
-    def head_norm_gate(self, o, H, Dv, weight, per_head, eps, gate, gate_col, activation):
+    def ssd_scan(self, src, x_col, b_col, c_col, H, G, N, P, steps, step_col, rates, step_bias, skip,
+                 state, batch, write):
+        """dt = softplus(steps[:, step_col + h] + step_bias[h]); S' = exp(-exp(rates[h]) dt) S +
+        dt B x^T; y = S'^T C + skip[h] x.  x [H, P] at x_col of src, B and C [G, N] at b_col and
+        c_col (head h reads group h // (H / G)).  The slot holds S as [H, P, N] from 0 on."""
+        T = src.shape[0]
+        x = src[:, x_col:x_col + H * P].float().view(T, H, P)
+        B = src[:, b_col:b_col + G * N].float().view(T, G, N).repeat_interleave(H // G, 1)
+        C = src[:, c_col:c_col + G * N].float().view(T, G, N).repeat_interleave(H // G, 1)
+        dt = torch.nn.functional.softplus(steps[:, step_col:step_col + H].float() + step_bias)
+        keep = torch.exp(-torch.exp(rates) * dt)
+        out = torch.empty(T, H, P)
+        for a, b, slot, fresh in self._sequences(batch):
+            kept = state[slot, :H * P * N].view(H, P, N)
+            S = torch.zeros(H, P, N) if fresh else kept.clone()
+            for t in range(a, b):
+                S = keep[t][:, None, None] * S + (dt[t][:, None] * x[t])[:, :, None] * B[t][:, None, :]
+                out[t] = torch.einsum("hpn,hn->hp", S, C[t]) + skip[:, None] * x[t]
+            if write:
+                kept.copy_(S)
+        return out.view(T, H * P)
+
+    def head_norm_gate(self, o, H, Dv, weight, per_head, eps, gate, gate_col, activation, gate_first=False):
         """Each head of o [T, H Dv] (float32) divided by its root mean square, times ``weight``
         ([H Dv] when ``per_head``, else [Dv] for every head), times sigmoid or silu of
         gate[:, gate_col:gate_col + H Dv]."""
         T = o.shape[0]
         x = o.view(T, H, Dv)
-        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
-        x = x * (weight.view(H, Dv) if per_head else weight)
         g = gate[:, gate_col:gate_col + H * Dv].float().view(T, H, Dv)
         g = torch.sigmoid(g) if activation == "sigmoid" else g * torch.sigmoid(g)
-        return (x * g).reshape(T, H * Dv).to(self.act_dtype)
+        if gate_first:              # the gate before the norm
+            x = x * g
+        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+        x = x * (weight.view(H, Dv) if per_head else weight)
+        if not gate_first:
+            x = x * g
+        return x.reshape(T, H * Dv).to(self.act_dtype)
 
     # -------------------------------------- attention with a norm over the projection
     def projnorm_rope_store(self, buf, H, G, D, Dv, q_gain, k_gain, eps, rot, tables, slots, k_cache,
@@ -312,6 +363,8 @@ class EmulatedOps:
         T = buf.shape[0]
 
         def normed(x, gain):
+            if gain is None:        # no norm over the projection
+                return x
             return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * gain
 
         def turned(x):
@@ -333,8 +386,8 @@ class EmulatedOps:
     def window_attention(self, q, q_col, nh, nkv, Dk, Dv, k_cache, v_cache, page_size, block_tables,
                          batch, scale, window, keep_first=0, slopes=None, sinks=None, gate=None,
                          gate_col=0):
-        if slopes is not None or sinks is not None or gate is not None or v_cache is None:
-            raise NotImplementedError("the emulated window attention has no bias, sink, gate or latent")
+        if slopes is not None or sinks is not None or gate is not None:
+            raise NotImplementedError("the emulated window attention has no bias, sink or gate")
         T = q.shape[0]
         g = nh // nkv
         out = torch.empty(T, nh * Dv, dtype=self.act_dtype)
@@ -352,12 +405,59 @@ class EmulatedOps:
             pages = block_tables[s].long()[k_pos // page_size]
             offs = k_pos % page_size
             k = _f(k_cache[pages, :, offs, :]).repeat_interleave(g, dim=1)
-            v = _f(v_cache[pages, :, :, offs]).repeat_interleave(g, dim=1)
+            if v_cache is None:     # the values are the first Dv channels of the key rows
+                v = k[..., :Dv]
+            else:
+                v = _f(v_cache[pages, :, :, offs]).repeat_interleave(g, dim=1)
             scores = torch.einsum("qhd,rhd->hqr", qs, k) * scale
             scores = scores.masked_fill(~vis[None], float("-inf"))
             o = torch.einsum("hqr,rhd->qhd", torch.softmax(scores, -1), v)
             out[a:b] = o.reshape(b - a, nh * Dv).to(self.act_dtype)
         return out
+
+    # ------------------------------------------------------- a cached latent
+    def slice_rmsnorm(self, buf, col, n, gain, eps):
+        x = _f(buf[:, col:col + n])
+        return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * gain).to(self.act_dtype)
+
+    def head_products(self, x, x_col, heads, x_head, A, y=None, y_col=0, y_head=None):
+        """y[t, h] = A[h] x[t, h]: head h's K values at column x_col + h * x_head of x, its N
+        results at column y_col + h * y_head of y."""
+        T = x.shape[0]
+        H, N, K = A.shape
+        y_head = N if y_head is None else y_head
+        if y is None:
+            y = torch.zeros(T, y_col + heads * y_head, dtype=self.act_dtype)
+        for h in range(heads):
+            xs = _f(x[:, x_col + h * x_head:x_col + h * x_head + K])
+            y[:, y_col + h * y_head:y_col + h * y_head + N] = (xs @ _f(A[h]).T).to(y.dtype)
+        return y
+
+    def latent_store(self, buf, nh, D, R, C, down_off, rot, gain, eps, tables, slots, k_cache,
+                     page_size, q_out, q_rows=None):
+        """The key row of a token: [RMS norm of buf[:, down_off:down_off + C] times gain | the next R
+        channels, the first ``rot`` of them turned in halves]; the last R channels of every query
+        head (in ``q_rows``, or in buf) turned the same way into q_out[t, h, C:]."""
+        T = buf.shape[0]
+        q_rows = buf if q_rows is None else q_rows
+        half = rot // 2
+
+        def turned(x):              # [..., R]
+            if not rot:
+                return x
+            c, s = tables.cos, tables.sin
+            while c.dim() < x.dim():
+                c, s = c[:, None], s[:, None]
+            a, b = x[..., :half], x[..., half:rot]
+            return torch.cat([a * c - b * s, b * c + a * s, x[..., rot:]], -1)
+        q = _f(q_rows[:, :nh * (D + R)]).view(T, nh, D + R)
+        q_out.view(T, nh, C + R)[:, :, C:] = turned(q[..., D:]).to(q_out.dtype)
+        if slots is not None:
+            c = _f(buf[:, down_off:down_off + C])
+            c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * gain
+            row = torch.cat([c, turned(_f(buf[:, down_off + C:down_off + C + R]))], -1)
+            page, off = (slots // page_size).long(), (slots % page_size).long()
+            k_cache[page, 0, off, :] = row.to(k_cache.dtype)
 
     # ------------------------------------------------------- routed experts
     def route_tokens(self, logits, experts, top):
@@ -367,19 +467,24 @@ class EmulatedOps:
         best = torch.topk(z, top, dim=-1, sorted=True)
         return best.indices.to(torch.int32), torch.softmax(best.values, -1)
 
-    def routed_experts(self, x, routing, w_gate_up, w_down, base=None):
-        """sum over a token's choices of share * down_e(silu(gate_e x) * up_e x) (+ base);
-        w_gate_up [E, 2 ff, width] holds an expert's gate rows before its up rows."""
+    def routed_experts(self, x, routing, w_gate_up, w_down, base=None, activation="silu", gated=True,
+                       base_gate=None, base_gate_col=0):
+        """sum over a token's choices of share * down_e(act(gate_e x) * up_e x) (+ base);
+        w_gate_up [E, 2 ff, width] holds an expert's gate rows before its up rows.  Not gated:
+        down_e(act(up_e x)) with w_gate_up [E, ff, width].  base_gate: base times the sigmoid of
+        base_gate[t, base_gate_col]."""
         chosen, shares = routing
         T = x.shape[0]
-        ff = w_gate_up.shape[1] // 2
+        ff = w_gate_up.shape[1] // 2 if gated else w_gate_up.shape[1]
         xf = _f(x)
         out = torch.zeros(T, w_down.shape[1]) if base is None else _f(base).clone()
+        if base_gate is not None:
+            out = out * torch.sigmoid(base_gate[:, base_gate_col].float())[:, None]
         for t in range(T):
             for e, s in zip(chosen[t].tolist(), shares[t].tolist()):
                 gu = _f(w_gate_up[e]) @ xf[t]
-                mid = (gu[:ff] * torch.sigmoid(gu[:ff]) * gu[ff:]).to(self.act_dtype).float()
-                out[t] += s * (_f(w_down[e]) @ mid)
+                mid = self._act(gu[:ff], activation) * gu[ff:] if gated else self._act(gu, activation)
+                out[t] += s * (_f(w_down[e]) @ mid.to(self.act_dtype).float())
         return out.to(self.act_dtype)
 
     # ------------------------------------------------------------- sampling
