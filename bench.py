@@ -126,9 +126,46 @@ def vekanex_configs(shape, layers):
     return vekanex, qwen
 
 
+# Layer sizes for --design futezen: the attention has the shape's heads; the latent attention a key/value
+# latent of 512 channels, a query latent of 1,536 and 64 rotated channels; the state-space mixer twice the
+# width in heads of 64 channels with states of 128 rows and 8 groups; the experts are Vekanex's.
+FUTEZEN_SHAPES = {
+    "3b": dict(q_rank=1536, kv_rank=512, rot_dim=64, ssm_heads=64, ssm_vdim=64, state=128, groups=8),
+    "7b": dict(q_rank=1536, kv_rank=512, rot_dim=64, ssm_heads=112, ssm_vdim=64, state=128, groups=8),
+}
+
+
+def futezen_configs(shape, layers):
+    """(Futezen config.json, Vekanex config.json) of equal size: Vekanex is the design nearest to it
+    (states in slots, routed experts with a shared one, norms on the sublayers' outputs, layers that run
+    again).  Futezen's layers come in the order latent attention (dense feed-forward), state-space mixer
+    (experts), attention (dense), latent attention (experts); with eight layers or more the first two run
+    twice."""
+    z, v, f = DESIGN_SHAPES[shape], VEKANEX_SHAPES[shape], FUTEZEN_SHAPES[shape]
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "router": {"experts": v["experts"], "top": v["top"]}, "expert": {"ff": v["expert_ff"]},
+           "shared": {"ff": v["shared_ff"]}}
+    lat = {"heads": z["heads"], "dim": z["dim"], "rot_dim": f["rot_dim"], "vdim": z["dim"], "q_rank": f["q_rank"],
+           "kv_rank": f["kv_rank"], "scale": (z["dim"] + f["rot_dim"]) ** -0.5,
+           "rot": {"base": 1e6, "dims": f["rot_dim"]}}
+    ssm = {"heads": f["ssm_heads"], "vdim": f["ssm_vdim"], "state": f["state"], "groups": f["groups"], "conv": 4,
+           "norm_groups": f["groups"]}
+    att = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+           "scale": z["dim"] ** -0.5, "rot": {"base": 1e4, "dims": z["dim"] // 2}}
+    order = [{"type": "latent_attention", "mixer": lat, "mlp": dense}, {"type": "mamba2", "mixer": ssm, "mlp": moe},
+             {"type": "attention", "mixer": att, "mlp": dense}, {"type": "latent_attention", "mixer": lat, "mlp": moe}]
+    futezen = {"architecture": "Futezen", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-5},
+               "torch_dtype": "bfloat16", "layers": [order[i % 4] for i in range(layers)]}
+    if layers >= 8:
+        futezen["layers"] = futezen["layers"][:layers - 2]
+        futezen["loop"] = {"start": 0, "stop": 2, "times": 2}
+    return futezen, vekanex_configs(shape, layers)[0]
+
+
 def compare_designs(args):
     """Prefill and decode throughput of the design named by --design beside the Qwen2 decoder of equal
-    size, at each of --design-shapes: one JSON line, tokens per second each."""
+    size (Futezen: beside the Vekanex decoder of equal size), at each of --design-shapes: one JSON line,
+    tokens per second each."""
     import torch
     import servelab_amd  # noqa: F401
     from servelab_amd.config import resolve_architecture
@@ -141,9 +178,11 @@ def compare_designs(args):
                       "prefill_chunk": args.prefill_chunk, "page_size": page}, "shapes": {}}
     for shape in args.design_shapes.split(","):
         row = {}
-        pair = vekanex_configs(shape, args.design_layers) if args.design == "vekanex" else \
+        other = "vekanex" if args.design == "futezen" else "qwen2"
+        pair = futezen_configs(shape, args.design_layers) if args.design == "futezen" else \
+            vekanex_configs(shape, args.design_layers) if args.design == "vekanex" else \
             design_configs(shape, args.design_layers, args.design_window)
-        for name, raw in zip((args.design, "qwen2"), pair):
+        for name, raw in zip((args.design, other), pair):
             cfg = resolve_architecture(raw).config_from_hf(raw, "")
             model = random_model_on_device(cfg, args.seed, args.dtype, "cuda:0")
             torch.cuda.synchronize()
@@ -154,8 +193,8 @@ def compare_designs(args):
                          "prefill_tok_s": round(args.prefill_tokens / pre_s, 1), "prefill_ms": round(pre_s * 1e3, 3)}
             del model
             torch.cuda.empty_cache()
-        row["decode_ratio"] = round(row[args.design]["decode_tok_s"] / row["qwen2"]["decode_tok_s"], 3)
-        row["prefill_ratio"] = round(row[args.design]["prefill_tok_s"] / row["qwen2"]["prefill_tok_s"], 3)
+        row["decode_ratio"] = round(row[args.design]["decode_tok_s"] / row[other]["decode_tok_s"], 3)
+        row["prefill_ratio"] = round(row[args.design]["prefill_tok_s"] / row[other]["prefill_tok_s"], 3)
         out["shapes"][shape] = row
     print(json.dumps(out))
     return 0
@@ -308,7 +347,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernel choice for the prompt products")
-    ap.add_argument("--design", default="", choices=["", "topelorn", "vekanex"],
+    ap.add_argument("--design", default="", choices=["", "topelorn", "vekanex", "futezen"],
                     help="instead of the default workload: prefill and decode throughput of this design "
                          "beside the Qwen2 decoder of equal size")
     ap.add_argument("--design-shapes", default="3b,7b", help="comma-separated: " + ", ".join(sorted(DESIGN_SHAPES)))
