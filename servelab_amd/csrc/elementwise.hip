@@ -48,6 +48,7 @@ struct __attribute__((aligned(16))) act8 { act_t v[8]; };
 struct __attribute__((aligned(16))) act8_half { act_t v[4]; };
 #endif
 
+template <int ACT>
 __global__ void silu_mul_block8_kernel(const act_t* __restrict__ gate_up, act_t* __restrict__ out,
                                        size_t groups) {
   for (size_t gidx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; gidx < groups;
@@ -60,7 +61,8 @@ __global__ void silu_mul_block8_kernel(const act_t* __restrict__ gate_up, act_t*
       const act8_half g = *(const act8_half*)(src + 4 * h), u = *(const act8_half*)(src + 8 + 4 * h);
       act8_half o;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) o.v[j] = g.v[j] / (1.f + expf(-g.v[j])) * u.v[j];
+      for (int j = 0; j < 4; ++j)
+        o.v[j] = (ACT == SL_ACT_SILU ? g.v[j] / (1.f + expf(-g.v[j])) : fmaxf(g.v[j], 0.f)) * u.v[j];
       *(act8_half*)(dst + 4 * h) = o;
     }
 #else
@@ -69,7 +71,7 @@ __global__ void silu_mul_block8_kernel(const act_t* __restrict__ gate_up, act_t*
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const float gf = to_f(g.v[j]);
-      o.v[j] = from_f<act_t>(gf / (1.f + __expf(-gf)) * to_f(u.v[j]));
+      o.v[j] = from_f<act_t>((ACT == SL_ACT_SILU ? gf / (1.f + __expf(-gf)) : fmaxf(gf, 0.f)) * to_f(u.v[j]));
     }
     *(act8*)dst = o;
 #endif
@@ -83,11 +85,14 @@ extern "C" const char* sl_gate_mul(const void* gate_up, void* out, int T, int I,
   SL_CHECK(block > 0 && I % block == 0, "silu_mul: the block must divide the width");
   if (T == 0) return nullptr;
   const size_t total = (size_t)T * I;
-  if (act == SL_ACT_SILU && block == 8 && ((uintptr_t)gate_up % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+  if (act != SL_ACT_RELU2 && block == 8 && ((uintptr_t)gate_up % 16) == 0 && ((uintptr_t)out % 16) == 0) {
     const size_t groups = total / 8;
     const size_t blocks = (groups + 255) / 256;
-    silu_mul_block8_kernel<<<(unsigned)(blocks < 262144 ? blocks : 262144), 256, 0, stream>>>(
-        (const act_t*)gate_up, (act_t*)out, groups);
+    const unsigned grid = (unsigned)(blocks < 262144 ? blocks : 262144);
+    if (act == SL_ACT_SILU)
+      silu_mul_block8_kernel<SL_ACT_SILU><<<grid, 256, 0, stream>>>((const act_t*)gate_up, (act_t*)out, groups);
+    else
+      silu_mul_block8_kernel<SL_ACT_RELU><<<grid, 256, 0, stream>>>((const act_t*)gate_up, (act_t*)out, groups);
     return sl_launch_status();
   }
   const int blocks = (int)((total + 255) / 256 < 65535 * 4 ? (total + 255) / 256 : 65535 * 4);

@@ -391,20 +391,37 @@ extern "C" const char* sl_latent_store(const void* qbuf, int q_stride, const voi
 
 // ---------------------------------------------------------------------------
 // The RMS norm of a slice of columns: out[t][c] = x[t][col + c] * rsqrt(mean_c x^2 + eps) * gain[c],
-// sums in float.  One wavefront per token (a latent has few channels).
+// sums in float.  One block per token: a thread asks for all its values at once (up to SLICE_KEEP of
+// them stay in registers, so the row makes one trip from memory) and the gains with them.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void slice_rmsnorm_kernel(const act_t* __restrict__ buf, int stride, int col, int n,
-                                                           const float* __restrict__ gain, float eps,
-                                                           act_t* __restrict__ out) {
+constexpr int SLICE_KEEP = 8;
+__global__ __launch_bounds__(256) void slice_rmsnorm_kernel(const act_t* __restrict__ buf, int stride, int col, int n,
+                                                            const float* __restrict__ gain, float eps,
+                                                            act_t* __restrict__ out) {
+  __shared__ float scratch[16];
   const size_t t = blockIdx.x;
   const act_t* x = buf + t * stride + col;
+  float keep[SLICE_KEEP], g[SLICE_KEEP];
   float ss = 0.f;
-  for (int d = threadIdx.x; d < n; d += 64) {
+#pragma unroll
+  for (int u = 0; u < SLICE_KEEP; ++u) {
+    const int d = threadIdx.x + u * 256;
+    keep[u] = d < n ? to_f(x[d]) : 0.f;
+    g[u] = d < n ? gain[d] : 0.f;
+  }
+#pragma unroll
+  for (int u = 0; u < SLICE_KEEP; ++u) ss += keep[u] * keep[u];
+  for (int d = threadIdx.x + SLICE_KEEP * 256; d < n; d += 256) {
     const float v = to_f(x[d]);
     ss += v * v;
   }
-  const float inv = 1.f / sqrtf(wave_sum(ss) / (float)n + eps);
-  for (int d = threadIdx.x; d < n; d += 64) out[t * n + d] = from_f<act_t>(to_f(x[d]) * inv * gain[d]);
+  const float inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)n + eps);
+#pragma unroll
+  for (int u = 0; u < SLICE_KEEP; ++u) {
+    const int d = threadIdx.x + u * 256;
+    if (d < n) out[t * n + d] = from_f<act_t>(keep[u] * inv * g[u]);
+  }
+  for (int d = threadIdx.x + SLICE_KEEP * 256; d < n; d += 256) out[t * n + d] = from_f<act_t>(to_f(x[d]) * inv * gain[d]);
 }
 
 extern "C" const char* sl_slice_rmsnorm(const void* buf, int stride, int col, int n, const float* gain, float eps,
@@ -412,6 +429,6 @@ extern "C" const char* sl_slice_rmsnorm(const void* buf, int stride, int col, in
   SL_CHECK(T >= 0 && n > 0 && col >= 0 && col + n <= stride, "slice_rmsnorm: the slice does not fit the rows");
   SL_CHECK(gain != nullptr, "slice_rmsnorm: the gain is required");
   if (T == 0) return nullptr;
-  slice_rmsnorm_kernel<<<T, 64, 0, stream>>>((const act_t*)buf, stride, col, n, gain, eps, (act_t*)out);
+  slice_rmsnorm_kernel<<<T, 256, 0, stream>>>((const act_t*)buf, stride, col, n, gain, eps, (act_t*)out);
   return sl_launch_status();
 }
