@@ -104,7 +104,19 @@ def _e():
     return config(48, 200, 1e-5, layers, (0, 2, 1))
 
 
-MODELS = {"A": _a(), "B": _b(), "C": _c(), "D": _d(), "E": _e()}
+def _f():
+    # wider layers: keys of 96 channels over a latent of 80, six heads on three kv heads, eight state-space
+    # heads in two groups, twelve experts; the two middle layers run twice
+    layers = [
+        latent(4, 32, 16, 48, 96, 80, 0.14, 1000000.0, dense(384)),
+        mamba2(8, 16, 64, 2, 3, 2, moe(12, 3, 64, 96)),
+        attention(6, 3, 64, 32, 0.125, 10000.0, 32, dense(384)),
+        latent(4, 32, 16, 48, 96, 80, 0.14, 1000000.0, moe(12, 3, 64, 96)),
+    ]
+    return config(256, 512, 1e-5, layers, (1, 3, 2))
+
+
+MODELS = {"A": _a(), "B": _b(), "C": _c(), "D": _d(), "E": _e(), "F": _f()}
 
 
 def tensor_shapes(cfg):

@@ -110,6 +110,24 @@ def test_every_way_of_cutting_gives_the_plain_logits(tmp_path, which, dtype):
         run_and_compare(tmp_path, folder, cfg, steps, ref, dtype, f"mixed{seed}", max_live=3, **kw)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompts_of_the_widest_model(tmp_path, dtype):
+    """Prompts of several hundred tokens: many pages a request, steps of enough rows for every product
+    kernel, the attentions on the matrix cores in bfloat16, the scan over many chunks."""
+    cfg = MODELS["F"]
+    folder, weights = write_folder(tmp_path, cfg, seed=16, tag="F")
+    requests = make_requests(cfg["vocab"], [613, 190], seed=12)
+    ref = reference(cfg, weights, requests)
+    kw = {"float32_bar": plain_float32_loss(cfg, weights, requests, ref)}
+    if dtype == "bfloat16":
+        kw["emulated"] = emulated_bfloat16(tmp_path, folder, cfg, requests, ref)
+    run_and_compare(tmp_path, folder, cfg, rs.whole(requests), ref, dtype, "whole", **kw)
+    run_and_compare(tmp_path, folder, cfg, rs.tail_decoded(requests, tail=40), ref, dtype, "decode", **kw)
+    run_and_compare(tmp_path, folder, cfg, rs.portions(requests, sizes=(100, 2, 255, 64, 7)), ref, dtype, "portions", **kw)
+    steps = rs.mixed(requests, {rid: len(t) - 30 for rid, t in requests.items()}, max_live=2, seed=5, max_portion=130)
+    run_and_compare(tmp_path, folder, cfg, steps, ref, dtype, "mixed", max_live=2, **kw)
+
+
 @pytest.mark.parametrize("page", [16, 32, 64])
 def test_pages_and_slots_are_used_again(tmp_path, page):
     """A pool no larger than the live requests need at their peak and three state slots for ten
