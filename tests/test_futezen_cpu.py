@@ -86,6 +86,22 @@ def test_missing_and_impossible_keys_name_themselves():
             FutezenConfig.from_hf(cfg)
 
 
+def test_keys_that_may_be_null_or_absent():
+    cfg = copy.deepcopy(MODELS["A"])
+    cfg["loop"] = None
+    cfg["layers"][1]["mlp"]["shared"] = None
+    cfg["layers"][2]["mlp"] = None
+    got = FutezenConfig.from_hf(cfg)
+    assert got.loop is None and got.order() == [0, 1, 2]
+    assert got.layers[1].mlp.shared_ff == 0 and got.layers[2].mlp is None
+    spec = build_model_spec(got)
+    names = set(spec.param_specs())
+    assert "l1.mlp.shared.up" not in names and "l1.mlp.shared.sg" not in names and "l1.mlp.router.b" in names
+    assert "l2.norm2" not in names and "l2.norm2b" not in names and "l2.norm1b" in names
+    cfg["loop"] = {"start": 1, "stop": 1, "times": 3}                # an empty stretch
+    assert FutezenConfig.from_hf(cfg).order() == [0, 1, 2]
+
+
 def test_cache_needs_and_run_list():
     spec = build_model_spec(FutezenConfig.from_hf(MODELS["A"]))
     assert len(spec.layers) == 3 and [c.layer for c in spec.run] == [0, 1, 2, 1, 2]
