@@ -3,6 +3,7 @@ from .layered import (BiasedAttentionConfig, DenseMlpConfig, LatentAttentionConf
                       TopelornConfig, WindowConfig)
 from .vekanex import VekanexConfig, VekanexLayer
 from .futezen import FutezenConfig, FutezenLayer
+from .vunadra import VunadraConfig, VunadraLayer
 from .engine import CacheConfig, SchedulerConfig, EngineConfig, PAGE_SIZES
 from .registry import (Architecture, register_architecture, registered_architectures,
                        resolve_architecture)

@@ -51,12 +51,24 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return t;
 }
 
-// Activations by number, as the calls of the kernel table pass them: 1 silu, 2 relu, 3 relu squared.
-enum { SL_ACT_SILU = 1, SL_ACT_RELU = 2, SL_ACT_RELU2 = 3 };
+// Activations by number, as the calls of the kernel table pass them: 1 silu, 2 relu, 3 relu squared,
+// 4 the tanh form of gelu; 5 only as a gate (sl_gated): clamped operands, a sigmoid of 1.702 g, up + 1.
+enum { SL_ACT_SILU = 1, SL_ACT_RELU = 2, SL_ACT_RELU2 = 3, SL_ACT_GELU_TANH = 4, SL_ACT_CLAMPED_SWISH = 5 };
 __device__ __forceinline__ float sl_act(float z, int act) {
   if (act == SL_ACT_SILU) return z / (1.f + expf(-z));
+  if (act == SL_ACT_GELU_TANH) return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
   const float r = fmaxf(z, 0.f);
   return act == SL_ACT_RELU2 ? r * r : r;
+}
+// A gate times its up product: act(g) * u; for the clamped form, with g' = min(g, limit) and
+// u' = clamp(u, -limit, limit): g' sigmoid(1.702 g') (u' + 1).
+__device__ __forceinline__ float sl_gated(float g, float u, int act, float limit) {
+  if (act == SL_ACT_CLAMPED_SWISH) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+  }
+  return sl_act(g, act) * u;
 }
 
 #define SL_CHECK(cond, msg) \

@@ -2,23 +2,50 @@
 #include "common.h"
 
 // ---------------------------------------------------------------- embedding
-// out[t, :] = float(table[ids[t], :]).  Replaces the embedding lookup of
+// out[t, :] = scale * float(table[ids[t], :]).  Replaces the embedding lookup of
 // servelab/parallel/tp_model.py:123; the residual stream it starts is float.
 __global__ void embed_kernel(const int* __restrict__ ids, const act_t* __restrict__ table,
-                             float* __restrict__ out, int H, int V) {
+                             float* __restrict__ out, int H, int V, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   id = id < 0 ? 0 : (id >= V ? V - 1 : id);     // the host rejects such ids; never fault
   const act_t* row = table + (size_t)id * H;
   float* o = out + (size_t)t * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f(row[i]);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = scale * to_f(row[i]);
 }
 
 extern "C" const char* sl_embed(const int* ids, const void* table, float* out, int T, int H,
-                                int V, hipStream_t stream) {
+                                int V, float scale, hipStream_t stream) {
   SL_CHECK(T >= 0 && H > 0 && V > 0, "embed: sizes must be positive");
   if (T == 0) return nullptr;
-  embed_kernel<<<T, 256, 0, stream>>>(ids, (const act_t*)table, out, H, V);
+  embed_kernel<<<T, 256, 0, stream>>>(ids, (const act_t*)table, out, H, V, scale);
+  return sl_launch_status();
+}
+
+// ------------------------------------------ two streams side by side, as rows
+// out[t] = [act(a[t] + delta[t]) | act(b[t])]: the float stream a (with what is still to be added
+// to it, if anything) and a second float stream b, rounded to the activation type, as the rows
+// [T, 2 H] of a product over both.
+__global__ void stream_pair_kernel(const float* __restrict__ a, const act_t* __restrict__ delta,
+                                   const float* __restrict__ b, act_t* __restrict__ out, int H, size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / (2 * (size_t)H);
+    const int c = (int)(idx - t * 2 * H);
+    float v;
+    if (c < H) v = a[t * H + c] + (delta != nullptr ? to_f(delta[t * H + c]) : 0.f);
+    else v = b[t * H + c - H];
+    out[idx] = from_f<act_t>(v);
+  }
+}
+
+extern "C" const char* sl_stream_pair(const float* a, const void* delta, const float* b, void* out, int T, int H,
+                                      hipStream_t stream) {
+  SL_CHECK(T >= 0 && H > 0, "stream_pair: sizes must be positive");
+  if (T == 0) return nullptr;
+  const size_t total = (size_t)T * 2 * H, blocks = (total + 255) / 256;
+  stream_pair_kernel<<<(unsigned)(blocks < 262144 ? blocks : 262144), 256, 0, stream>>>(
+      a, (const act_t*)delta, b, (act_t*)out, H, total);
   return sl_launch_status();
 }
 
@@ -48,6 +75,12 @@ struct __attribute__((aligned(16))) act8 { act_t v[8]; };
 struct __attribute__((aligned(16))) act8_half { act_t v[4]; };
 #endif
 
+template <int ACT> __device__ __forceinline__ float gate_of(float g) {
+  if (ACT == SL_ACT_SILU) return g / (1.f + __expf(-g));
+  if (ACT == SL_ACT_RELU) return fmaxf(g, 0.f);
+  return sl_act(g, ACT);
+}
+
 template <int ACT>
 __global__ void silu_mul_block8_kernel(const act_t* __restrict__ gate_up, act_t* __restrict__ out,
                                        size_t groups) {
@@ -62,7 +95,7 @@ __global__ void silu_mul_block8_kernel(const act_t* __restrict__ gate_up, act_t*
       act8_half o;
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        o.v[j] = (ACT == SL_ACT_SILU ? g.v[j] / (1.f + expf(-g.v[j])) : fmaxf(g.v[j], 0.f)) * u.v[j];
+        o.v[j] = (ACT == SL_ACT_SILU ? g.v[j] / (1.f + expf(-g.v[j])) : sl_act(g.v[j], ACT)) * u.v[j];
       *(act8_half*)(dst + 4 * h) = o;
     }
 #else
@@ -71,7 +104,7 @@ __global__ void silu_mul_block8_kernel(const act_t* __restrict__ gate_up, act_t*
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const float gf = to_f(g.v[j]);
-      o.v[j] = from_f<act_t>((ACT == SL_ACT_SILU ? gf / (1.f + __expf(-gf)) : fmaxf(gf, 0.f)) * to_f(u.v[j]));
+      o.v[j] = from_f<act_t>(gate_of<ACT>(gf) * to_f(u.v[j]));
     }
     *(act8*)dst = o;
 #endif
@@ -81,7 +114,7 @@ __global__ void silu_mul_block8_kernel(const act_t* __restrict__ gate_up, act_t*
 extern "C" const char* sl_gate_mul(const void* gate_up, void* out, int T, int I, int block, int act,
                                    hipStream_t stream) {
   SL_CHECK(T >= 0 && I > 0, "silu_mul: sizes must be positive");
-  SL_CHECK(act >= SL_ACT_SILU && act <= SL_ACT_RELU2, "gate_mul: unknown activation");
+  SL_CHECK(act >= SL_ACT_SILU && act <= SL_ACT_GELU_TANH, "gate_mul: unknown activation");
   SL_CHECK(block > 0 && I % block == 0, "silu_mul: the block must divide the width");
   if (T == 0) return nullptr;
   const size_t total = (size_t)T * I;
@@ -91,6 +124,8 @@ extern "C" const char* sl_gate_mul(const void* gate_up, void* out, int T, int I,
     const unsigned grid = (unsigned)(blocks < 262144 ? blocks : 262144);
     if (act == SL_ACT_SILU)
       silu_mul_block8_kernel<SL_ACT_SILU><<<grid, 256, 0, stream>>>((const act_t*)gate_up, (act_t*)out, groups);
+    else if (act == SL_ACT_GELU_TANH)
+      silu_mul_block8_kernel<SL_ACT_GELU_TANH><<<grid, 256, 0, stream>>>((const act_t*)gate_up, (act_t*)out, groups);
     else
       silu_mul_block8_kernel<SL_ACT_RELU><<<grid, 256, 0, stream>>>((const act_t*)gate_up, (act_t*)out, groups);
     return sl_launch_status();
@@ -113,7 +148,7 @@ __global__ void activate_kernel(const act_t* __restrict__ x, act_t* __restrict__
 
 extern "C" const char* sl_activate(const void* x, void* out, long long n, int act, hipStream_t stream) {
   SL_CHECK(n >= 0, "activate: the count must not be negative");
-  SL_CHECK(act >= SL_ACT_SILU && act <= SL_ACT_RELU2, "activate: unknown activation");
+  SL_CHECK(act >= SL_ACT_SILU && act <= SL_ACT_GELU_TANH, "activate: unknown activation");
   if (n == 0) return nullptr;
   const size_t blocks = ((size_t)n + 255) / 256;
   activate_kernel<<<(unsigned)(blocks < 262144 ? blocks : 262144), 256, 0, stream>>>((const act_t*)x, (act_t*)out,
@@ -122,26 +157,26 @@ extern "C" const char* sl_activate(const void* x, void* out, long long n, int ac
 }
 
 // ------------------------------------------------------------ rotary tables
-// cos/sin[t, j] of angle float(pos[t]) * inv_freq[j], float32 with the
+// magnitude * cos/sin[t, j] of angle float(pos[t]) * inv_freq[j], float32 with the
 // accurate cosf/sinf.  Once per step; every layer reads the same table.
 __global__ void rope_tables_kernel(const int* __restrict__ pos, const float* __restrict__ inv_freq,
                                    float* __restrict__ cosv, float* __restrict__ sinv,
-                                   int half, int total) {
+                                   int half, int total, float magnitude) {
   const int idx = blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const int t = idx / half, j = idx - t * half;
   const float ang = (float)pos[t] * inv_freq[j];
-  cosv[idx] = cosf(ang);
-  sinv[idx] = sinf(ang);
+  cosv[idx] = cosf(ang) * magnitude;
+  sinv[idx] = sinf(ang) * magnitude;
 }
 
 extern "C" const char* sl_rope_tables(const int* pos, const float* inv_freq, float* cosv,
-                                      float* sinv, int T, int half, hipStream_t stream) {
+                                      float* sinv, int T, int half, float magnitude, hipStream_t stream) {
   SL_CHECK(T >= 0 && half > 0, "rope_tables: sizes must be positive");
   if (T == 0) return nullptr;
   const int total = T * half;
   rope_tables_kernel<<<(total + 255) / 256, 256, 0, stream>>>(pos, inv_freq, cosv, sinv, half,
-                                                              total);
+                                                              total, magnitude);
   return sl_launch_status();
 }
 

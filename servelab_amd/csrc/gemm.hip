@@ -743,6 +743,10 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
             gsum *= inv;
             usum *= inv;
           }
+          if (bias != nullptr) {                  // (the bias lies as the rows do: 8 gates, their 8 ups)
+            gsum += bias[tile * 16 + j];
+            usum += bias[tile * 16 + 8 + j];
+          }
           const size_t at = F.y_tiled ? (size_t)(n / 32) * (M * 32) + m * 32 + n % 32 : (size_t)m * (N / 2) + n;
           ((__bf16*)y)[at] = (__bf16)(sl_act(gsum, F.gate_act) * usum);
         }
@@ -821,8 +825,8 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
   SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: sizes must be positive");
   SL_CHECK(M <= 16, "gemm_skinny: at most 16 rows");
   SL_CHECK(K % 32 == 0, "gemm_skinny: K must be a multiple of 32");
-  SL_CHECK(!gated || (N % 16 == 0 && bias == nullptr && !out_f32),
-           "gemm_skinny: the gated form needs N % 16 == 0, no bias, activation output");
+  SL_CHECK(!gated || (N % 16 == 0 && !out_f32),
+           "gemm_skinny: the gated form needs N % 16 == 0, activation output");
   SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wt % 16) == 0,
            "gemm_skinny: x and W must be 16-byte aligned");
   const bool consumer = in_parts != nullptr, producer = resid != nullptr;
@@ -985,6 +989,10 @@ __global__ __launch_bounds__(512) void gemm_resident_kernel(
           }
           gsum *= inv;
           usum *= inv;
+          if (bias != nullptr) {
+            gsum += bias[tile * 16 + j];
+            usum += bias[tile * 16 + 8 + j];
+          }
           const size_t at = F.y_tiled ? (size_t)(col / 32) * (M * 32) + m * 32 + col % 32 : (size_t)m * (N / 2) + col;
           ((__bf16*)y)[at] = (__bf16)(sl_act(gsum, F.gate_act) * usum);
         }
@@ -1044,8 +1052,8 @@ extern "C" const char* sl_gemm_resident(const void* x, const void* wt, const flo
   SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_resident: sizes must be positive");
   SL_CHECK(M <= 16, "gemm_resident: at most 16 rows");
   SL_CHECK(sl_gemm_resident_parts(K) > 0, "gemm_resident: no kernel for rows of this length");
-  SL_CHECK(!gated || (N % 16 == 0 && bias == nullptr && !out_f32),
-           "gemm_resident: the gated form needs N % 16 == 0, no bias, activation output");
+  SL_CHECK(!gated || (N % 16 == 0 && !out_f32),
+           "gemm_resident: the gated form needs N % 16 == 0, activation output");
   SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wt % 16) == 0,
            "gemm_resident: x and W must be 16-byte aligned");
   SL_CHECK(in_parts != nullptr && in_nparts > 0 && eps > 0.f, "gemm_resident: needs parts and eps");
@@ -1209,6 +1217,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(
             gsum += red[wv][b][m_local + 16 * (j / 4)][j % 4];
             usum += red[wv][b][m_local + 16 * (2 + j / 4)][j % 4];
           }
+          if (bias != nullptr) {
+            gsum += bias[(tile0 + t) * 16 + j];
+            usum += bias[(tile0 + t) * 16 + 8 + j];
+          }
           ((__bf16*)y)[(size_t)m * (N / 2) + n] = (__bf16)(sl_act(gsum, gate_act) * usum);
         }
       }
@@ -1235,8 +1247,8 @@ extern "C" const char* sl_gemm_wide(const void* x, const void* wt, const float* 
   SL_CHECK(M > 0 && N > 0 && K > 0, "gemm_wide: sizes must be positive");
   SL_CHECK(M <= 64, "gemm_wide: at most 64 rows");
   SL_CHECK(K % 32 == 0, "gemm_wide: K must be a multiple of 32");
-  SL_CHECK(!gated || (N % 16 == 0 && bias == nullptr && !out_f32),
-           "gemm_wide: the gated form needs N % 16 == 0, no bias, activation output");
+  SL_CHECK(!gated || (N % 16 == 0 && !out_f32),
+           "gemm_wide: the gated form needs N % 16 == 0, activation output");
   SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wt % 16) == 0,
            "gemm_wide: x and W must be 16-byte aligned");
   const dim3 grid(((N + 15) / 16 + 1) / 2);
@@ -1479,8 +1491,12 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
           __bf16* o = (__bf16*)y + (size_t)m * (N / 2) + tile_of[t] * 8 + 4 * gq;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float g = acc[t][b][r];
-            o[r] = (__bf16)(sl_act(g, gated) * up[r]);
+            float g = acc[t][b][r], u = up[r];
+            if (bias != nullptr) {
+              g += bias[n + r];
+              u += bias[n + 8 + r];
+            }
+            o[r] = (__bf16)(sl_act(g, gated) * u);
           }
         }
         continue;
@@ -1545,8 +1561,8 @@ extern "C" const char* sl_gemm_mid(const void* x, const void* wt, const float* b
   SL_CHECK(ks >= 1 && ks <= 16 && ks <= K / 32, "gemm_mid: ks must be in 1..16 and <= K / 32");
   SL_CHECK(ks == 1 || part != nullptr, "gemm_mid: a split of K needs the partial buffer");
   SL_CHECK(y != nullptr || ks > 1, "gemm_mid: no output");
-  SL_CHECK(!gated || (ks == 1 && N % 16 == 0 && bias == nullptr && !out_f32),
-           "gemm_mid: the gated form needs ks == 1, N % 16 == 0, no bias, activation output");
+  SL_CHECK(!gated || (ks == 1 && N % 16 == 0 && !out_f32),
+           "gemm_mid: the gated form needs ks == 1, N % 16 == 0, activation output");
   SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wt % 16) == 0,
            "gemm_mid: x and W must be 16-byte aligned");
   const int ntiles = (N + 15) / 16;

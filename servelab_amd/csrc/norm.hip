@@ -445,3 +445,16 @@ extern "C" const char* sl_softcap(float* x, float cap, long long n, hipStream_t 
   softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, cap, (size_t)n);
   return sl_launch_status();
 }
+
+// x *= factor in place on float values (logits).
+__global__ void scale_kernel(float* __restrict__ x, float factor, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] *= factor;
+}
+
+extern "C" const char* sl_scale(float* x, float factor, long long n, hipStream_t stream) {
+  SL_CHECK(n >= 0, "scale: the count must not be negative");
+  if (n == 0) return nullptr;
+  scale_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, factor, (size_t)n);
+  return sl_launch_status();
+}

@@ -100,6 +100,7 @@ struct ShortConv {
   const int* slots;
   int unit_heads, unit_dim, scaled_heads;
   float unit_eps, scale;
+  int silu;                  // 0: the convolution's sum leaves as it is
   float* out;                // [T][C]
 };
 
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(64) void short_conv_kernel(const ShortConv a) {
         else x = fresh ? 0.f : past[(size_t)(back + idx) * a.C + c];
         acc += a.w[(size_t)c * a.taps + j] * x;
       }
-      y[u] = acc * sigmoidf_(acc);
+      y[u] = a.silu ? acc * sigmoidf_(acc) : acc;
       ss += y[u] * y[u];
     }
   }
@@ -174,7 +175,7 @@ extern "C" const char* sl_short_conv(const float* buf, int stride, int col, int 
                                      const float* bias, float* state, long long state_stride, int state_off, const int* cu_q,
                                      const int* positions, const int* tok_seq, const int* slots, int S, int T,
                                      int write, int unit_heads, int unit_dim, float unit_eps, int scaled_heads,
-                                     float scale, float* out, hipStream_t stream) {
+                                     float scale, int silu, float* out, hipStream_t stream) {
   SL_CHECK(T >= 0 && S >= 0 && C > 0 && taps >= 1 && taps <= 64, "short_conv: sizes must be positive, taps <= 64");
   SL_CHECK(col >= 0 && col + C <= stride, "short_conv: the channels do not fit the rows");
   SL_CHECK(unit_heads >= 0 && (unit_heads == 0 || (unit_dim >= 1 && unit_dim <= 256)) &&
@@ -184,7 +185,7 @@ extern "C" const char* sl_short_conv(const float* buf, int stride, int col, int 
            "short_conv: the last inputs do not fit the state slot");
   if (T == 0) return nullptr;
   const ShortConv a{buf, stride, col, C, taps, w, bias, state, state_stride, state_off, cu_q, positions, tok_seq,
-                    slots, unit_heads, unit_dim, scaled_heads, unit_eps, scale, out};
+                    slots, unit_heads, unit_dim, scaled_heads, unit_eps, scale, silu, out};
   const int rest = C - unit_heads * unit_dim;
   short_conv_kernel<<<dim3(T, unit_heads + (rest + 255) / 256), 64, 0, stream>>>(a);
   if (write && taps > 1) short_conv_state_kernel<<<dim3(S, (C + 255) / 256), 256, 0, stream>>>(a, S);
@@ -575,12 +576,15 @@ extern "C" const char* sl_head_norm_gate(const float* o, int T, int H, int Dv, c
 // buf row: q [H][D], k [G][D], v [G][Dv] (float).  q and k are divided by the root mean square of
 // all their heads together and multiplied by a gain of that size (no gains: no norm), then the first `rot` channels
 // of every head turn in halves (channel i with i + rot / 2, angle of cos/sin column i).  q leaves
-// in the activation type; k and v go to the token's place in the pages.  One block per token.
+// in the activation type; k and v go to the token's place in the pages.  The values lie at column
+// v_col of the row (behind k: (H + G) D; at H D the values are the keys as the projection left
+// them, before norm and rotation).  One block per token.
 __global__ void projnorm_rope_store_kernel(const float* __restrict__ buf, int stride, int H, int G, int D, int Dv,
                                            const float* __restrict__ qw, const float* __restrict__ kw, float eps,
                                            int rot, const float* __restrict__ cosv, const float* __restrict__ sinv,
                                            const int* __restrict__ slots, act_t* __restrict__ kc,
-                                           act_t* __restrict__ vc, int page, act_t* __restrict__ q_out) {
+                                           act_t* __restrict__ vc, int page, act_t* __restrict__ q_out,
+                                           int v_col) {
   __shared__ float scratch[16];
   const size_t t = blockIdx.x;
   const float* row = buf + t * stride;
@@ -618,21 +622,22 @@ __global__ void projnorm_rope_store_kernel(const float* __restrict__ buf, int st
   }
   if (slots != nullptr)
     for (int e = threadIdx.x; e < nv; e += blockDim.x)
-      vc[((pg * G + e / Dv) * Dv + e % Dv) * page + off] = from_f<act_t>(row[nq + nk + e]);
+      vc[((pg * G + e / Dv) * Dv + e % Dv) * page + off] = from_f<act_t>(row[v_col + e]);
 }
 
 extern "C" const char* sl_projnorm_rope_store(const float* buf, int stride, int T, int H, int G, int D, int Dv,
                                               const float* qw, const float* kw, float eps, int rot,
                                               const float* cosv, const float* sinv, const int* slots, void* kc,
-                                              void* vc, int page, void* q_out, hipStream_t stream) {
+                                              void* vc, int page, void* q_out, int v_col, hipStream_t stream) {
   SL_CHECK(T >= 0 && H > 0 && G > 0 && D > 0 && Dv > 0 && page > 0, "projnorm_rope_store: sizes must be positive");
-  SL_CHECK((long long)(H + G) * D + (long long)G * Dv <= stride, "projnorm_rope_store: q, k and v do not fit the rows");
+  SL_CHECK((long long)(H + G) * D <= stride && v_col >= 0 && v_col + (long long)G * Dv <= stride,
+           "projnorm_rope_store: q, k and v do not fit the rows");
   SL_CHECK(rot >= 0 && rot % 2 == 0 && rot <= D, "projnorm_rope_store: the rotated width must be even and within a head");
   SL_CHECK(rot == 0 || (cosv != nullptr && sinv != nullptr), "projnorm_rope_store: cos and sin are missing");
   SL_CHECK((qw == nullptr) == (kw == nullptr), "projnorm_rope_store: both gains or neither");
   SL_CHECK(slots == nullptr || (kc != nullptr && vc != nullptr), "projnorm_rope_store: pages are missing");
   if (T == 0) return nullptr;
   projnorm_rope_store_kernel<<<T, 256, 0, stream>>>(buf, stride, H, G, D, Dv, qw, kw, eps, rot, cosv, sinv, slots,
-                                                    (act_t*)kc, (act_t*)vc, page, (act_t*)q_out);
+                                                    (act_t*)kc, (act_t*)vc, page, (act_t*)q_out, v_col);
   return sl_launch_status();
 }

@@ -1,5 +1,8 @@
 // Routed experts: every token goes through the `top` experts with the largest router logits,
-// weighted by the softmax over those logits only.
+// weighted by the softmax over those logits only; or (shares over all experts) with the largest
+// softmax shares plus a correction per expert, weighted by their shares, divided by their sum
+// and multiplied by a constant.  The last experts may be ones without matrices that hand their
+// input through.
 //
 //   route       per token the chosen experts and their shares (float), one wavefront a token
 //   group       the step's (token, choice) pairs sorted by expert, on the device: where each
@@ -20,11 +23,24 @@
 
 // ------------------------------------------------------------------ route
 // One wavefront per token.  Largest first; among equal logits the lower index wins.
+// over_all: the numbers compared are softmax(z)[e] + correction[e] over all E, and a chosen
+// expert's share is softmax(z)[e] / (sum over the chosen + 1e-20) * scale.
 __global__ __launch_bounds__(64) void route_kernel(const float* __restrict__ logits, int stride, int E, int top,
-                                                   int* __restrict__ chosen, float* __restrict__ shares) {
+                                                   int* __restrict__ chosen, float* __restrict__ shares,
+                                                   int over_all, const float* __restrict__ correction,
+                                                   float scale) {
   const size_t t = blockIdx.x;
   const int lane = threadIdx.x;
   const float* z = logits + t * stride;
+  float zmax = 0.f, inv_sum = 1.f;
+  if (over_all) {
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    zmax = wave_max(mx);
+    float sm = 0.f;
+    for (int e = lane; e < E; e += 64) sm += expf(z[e] - zmax);
+    inv_sum = 1.f / wave_sum(sm);
+  }
   unsigned long long taken = 0ull;             // bit u: element lane + 64 u is chosen already (E <= 4096)
   float mine = 0.f;                            // lane k keeps the k-th largest logit
   int mine_e = 0;
@@ -32,7 +48,8 @@ __global__ __launch_bounds__(64) void route_kernel(const float* __restrict__ log
     float best = -INFINITY;
     int at = 0x7fffffff;
     for (int u = 0, e = lane; e < E; ++u, e += 64) {
-      const float v = z[e];
+      float v = z[e];
+      if (over_all) v = expf(v - zmax) * inv_sum + (correction != nullptr ? correction[e] : 0.f);
       if (!((taken >> u) & 1ull) && (v > best || (v == best && e < at))) {
         best = v;
         at = e;
@@ -53,6 +70,15 @@ __global__ __launch_bounds__(64) void route_kernel(const float* __restrict__ log
       mine_e = at;
     }
   }
+  if (over_all) {
+    const float w = lane < top ? expf(z[mine_e] - zmax) * inv_sum : 0.f;
+    const float sum = wave_sum(w);
+    if (lane < top) {
+      chosen[t * top + lane] = mine_e;
+      shares[t * top + lane] = w / (sum + 1e-20f) * scale;
+    }
+    return;
+  }
   const float top1 = __shfl(mine, 0, SL_WAVE);
   const float w = lane < top ? expf(mine - top1) : 0.f;
   const float sum = wave_sum(w);
@@ -66,7 +92,8 @@ __global__ __launch_bounds__(64) void route_kernel(const float* __restrict__ log
 // One workgroup sorts the n = tokens * top pairs by expert (counting sort in LDS).
 //   order[place] = pair (token * top + choice);  place_of[pair] = place
 //   tiles[i] = {expert, first row, rows} for i < tiles in use; rows 0 beyond
-__global__ __launch_bounds__(1024) void group_kernel(const int* __restrict__ chosen, int n, int E, int max_tiles,
+// Experts from E_real on have no matrices: their pairs get places but no tiles.
+__global__ __launch_bounds__(1024) void group_kernel(const int* __restrict__ chosen, int n, int E, int E_real, int max_tiles,
                                                      int tile_rows, int* __restrict__ order,
                                                      int* __restrict__ place_of, int* __restrict__ tiles) {
   extern __shared__ int sh[];
@@ -89,11 +116,11 @@ __global__ __launch_bounds__(1024) void group_kernel(const int* __restrict__ cho
       start[e] = rows;
       tile0[e] = nt;
       rows += count[e];
-      nt += (count[e] + tile_rows - 1) / tile_rows;
+      if (e < E_real) nt += (count[e] + tile_rows - 1) / tile_rows;
     }
   }
   __syncthreads();
-  for (int e = tid; e < E; e += blockDim.x) {
+  for (int e = tid; e < E_real; e += blockDim.x) {
     const int c = count[e];
     for (int i = 0; i * tile_rows < c; ++i) {
       int* tl = tiles + 3 * (tile0[e] + i);
@@ -114,15 +141,18 @@ __global__ __launch_bounds__(1024) void group_kernel(const int* __restrict__ cho
 
 extern "C" const char* sl_route_tokens(const float* logits, int stride, int T, int E, int top, int* chosen,
                                        float* shares, int* order, int* place_of, int* tiles, int max_tiles,
-                                       int tile_rows, hipStream_t stream) {
+                                       int tile_rows, int over_all, const float* correction, float scale,
+                                       int E_real, hipStream_t stream) {
   SL_CHECK(T >= 0 && E >= 1 && E <= 4096 && top >= 1 && top <= 64 && top <= E && E <= stride,
            "route_tokens: at most 4096 experts within the rows, at most 64 choices");
+  SL_CHECK(E_real >= 0 && E_real <= E && (over_all || correction == nullptr),
+           "route_tokens: the experts with matrices are the first of all; a correction needs shares over all");
   SL_CHECK(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "route_tokens: row tiles hold 16, 64 or 128 rows");
   SL_CHECK(max_tiles >= ((long long)T * top + tile_rows - 1) / tile_rows + E, "route_tokens: too few tile entries");
   if (T == 0) return nullptr;
-  route_kernel<<<T, 64, 0, stream>>>(logits, stride, E, top, chosen, shares);
-  group_kernel<<<1, 1024, 3 * E * sizeof(int), stream>>>(chosen, T * top, E, max_tiles, tile_rows, order, place_of,
-                                                         tiles);
+  route_kernel<<<T, 64, 0, stream>>>(logits, stride, E, top, chosen, shares, over_all, correction, scale);
+  group_kernel<<<1, 1024, 3 * E * sizeof(int), stream>>>(chosen, T * top, E, E_real, max_tiles, tile_rows, order,
+                                                         place_of, tiles);
   return sl_launch_status();
 }
 
@@ -140,6 +170,7 @@ struct Grouped {
   act_t* out_act;            // gated and activated: [rows][N]
   float* out_f32;            // plain: [rows][N]
   int act;                   // the activation (common.h); 0 with out_f32
+  float limit;               // the clamped gate's bound
   int max_tiles, col_blocks; // the matrix-core kernels' launch: max_tiles x col_blocks workgroups in a row
 };
 
@@ -208,7 +239,7 @@ __global__ __launch_bounds__(256) void grouped_product_kernel(const Grouped a) {
     const int n = n0 + l + 16 * u;
     if (n >= a.N) continue;
     const size_t at = (size_t)(row0 + r) * a.N + n;
-    if (GATED) a.out_act[at] = from_f<act_t>(sl_act(acc[u], a.act) * acc2[u]);
+    if (GATED) a.out_act[at] = from_f<act_t>(sl_gated(acc[u], acc2[u], a.act, a.limit));
     else if (a.act) a.out_act[at] = from_f<act_t>(sl_act(acc[u], a.act));
     else a.out_f32[at] = acc[u];
   }
@@ -292,7 +323,7 @@ __global__ __launch_bounds__(64 * WR * WC) void grouped_product_mfma_kernel(cons
       if (GATED) {
         rt_bf16x4 r;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) r[c] = (__bf16)(sl_act(acc[v][u][c], a.act) * acc2[v][u][c]);
+        for (int c = 0; c < 4; ++c) r[c] = (__bf16)sl_gated(acc[v][u][c], acc2[v][u][c], a.act, a.limit);
         *(rt_bf16x4*)(a.out_act + at + 16 * u) = r;
       } else if (a.act) {
         rt_bf16x4 r;
@@ -408,7 +439,7 @@ __global__ __launch_bounds__(256, 2) void grouped_product_staged_kernel(const Gr
       if (GATED) {
         rt_bf16x4 r;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) r[c] = (__bf16)(sl_act(acc[v][u][c], a.act) * acc[v][NU + u][c]);
+        for (int c = 0; c < 4; ++c) r[c] = (__bf16)sl_gated(acc[v][u][c], acc[v][NU + u][c], a.act, a.limit);
         *(rt_bf16x4*)(a.out_act + at + 16 * u) = r;
       } else if (a.act) {
         rt_bf16x4 r;
@@ -425,15 +456,16 @@ __global__ __launch_bounds__(256, 2) void grouped_product_staged_kernel(const Gr
 
 extern "C" const char* sl_grouped_product(const void* x, const int* order, int top, const void* w, const int* tiles,
                                           int w_tiled, int max_tiles, int tile_rows, int N, int K, int gated,
-                                          int act, void* out, hipStream_t stream) {
+                                          int act, float limit, void* out, hipStream_t stream) {
   // gated: act(gate) * up into the activation type; else act != 0: act(W x) into the activation type;
   // else plain float sums
   SL_CHECK(max_tiles >= 0 && N > 0 && K > 0 && top >= 1, "grouped_product: sizes must be positive");
-  SL_CHECK(act >= 0 && act <= SL_ACT_RELU2 && (!gated || act), "grouped_product: unknown activation, or a gate without one");
+  SL_CHECK(act >= 0 && act <= SL_ACT_CLAMPED_SWISH && (!gated || act) && (gated || act != SL_ACT_CLAMPED_SWISH),
+           "grouped_product: unknown activation, a gate without one, or the clamped form without a gate");
   SL_CHECK(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "grouped_product: row tiles hold 16, 64 or 128 rows");
   if (max_tiles == 0) return nullptr;
   Grouped a{(const act_t*)x, order, top, (const act_t*)w, w_tiled, tiles, tile_rows / RT_ROWS, N, K,
-            act ? (act_t*)out : nullptr, act ? nullptr : (float*)out, act, max_tiles, 1};
+            act ? (act_t*)out : nullptr, act ? nullptr : (float*)out, act, limit, max_tiles, 1};
 #if !defined(SL_F32)
   if (K % 32 == 0 && N % 16 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0) {
     // (a one-dimensional launch of max_tiles x col_blocks workgroups, rounded up to the eight dies)
@@ -466,18 +498,22 @@ extern "C" const char* sl_grouped_product(const void* x, const int* order, int t
 
 // ------------------------------------------------------------------ combine
 // out[t] = g[t] base[t] + sum_k shares[t][k] * y[place_of[t top + k]], float sums, choices in their order;
-// g[t] = sigmoid(base_gate[t * gate_stride]) when base_gate is given, else 1.
+// g[t] = sigmoid(base_gate[t * gate_stride]) when base_gate is given, else 1.  A choice from
+// E_real on (chosen given) is an expert that hands its input through: it adds share * x[t].
 __global__ __launch_bounds__(256) void routed_combine_kernel(const float* __restrict__ y,
                                                              const int* __restrict__ place_of,
                                                              const float* __restrict__ shares, int top,
                                                              const act_t* __restrict__ base,
                                                              const float* __restrict__ base_gate, int gate_stride,
-                                                             int H, act_t* __restrict__ out) {
+                                                             int H, act_t* __restrict__ out,
+                                                             const int* __restrict__ chosen, int E_real,
+                                                             const act_t* __restrict__ x) {
   __shared__ int place[64];
   __shared__ float share[64];
   const size_t t = blockIdx.x;
   if (threadIdx.x < top) {
-    place[threadIdx.x] = place_of[t * top + threadIdx.x];
+    const bool through = chosen != nullptr && chosen[t * top + threadIdx.x] >= E_real;
+    place[threadIdx.x] = through ? -1 : place_of[t * top + threadIdx.x];
     share[threadIdx.x] = shares[t * top + threadIdx.x];
   }
   __syncthreads();
@@ -485,16 +521,20 @@ __global__ __launch_bounds__(256) void routed_combine_kernel(const float* __rest
   if (c >= H) return;
   float v = base != nullptr ? to_f(base[t * H + c]) : 0.f;
   if (base_gate != nullptr) v *= 1.f / (1.f + expf(-base_gate[t * gate_stride]));
-  for (int k = 0; k < top; ++k) v += share[k] * y[(size_t)place[k] * H + c];
+  for (int k = 0; k < top; ++k)
+    v += share[k] * (place[k] < 0 ? to_f(x[t * H + c]) : y[(size_t)place[k] * H + c]);
   out[t * H + c] = from_f<act_t>(v);
 }
 
 extern "C" const char* sl_routed_combine(const float* y, const int* place_of, const float* shares, int T, int top,
                                          const void* base, const float* base_gate, int gate_stride, int H,
-                                         void* out, hipStream_t stream) {
+                                         void* out, const int* chosen, int E_real, const void* x,
+                                         hipStream_t stream) {
   SL_CHECK(T >= 0 && top >= 1 && top <= 64 && H > 0, "routed_combine: sizes must be positive, at most 64 choices");
+  SL_CHECK(chosen == nullptr || x != nullptr, "routed_combine: experts that hand their input through need the input");
   if (T == 0) return nullptr;
   routed_combine_kernel<<<dim3(T, (H + 255) / 256), 256, 0, stream>>>(y, place_of, shares, top, (const act_t*)base,
-                                                                    base_gate, gate_stride, H, (act_t*)out);
+                                                                    base_gate, gate_stride, H, (act_t*)out,
+                                                                    chosen, E_real, (const act_t*)x);
   return sl_launch_status();
 }

@@ -15,6 +15,7 @@ struct WindowAttention {
   const int* positions;      // [tokens]
   int nh, nkv, Dk, Dv, page;
   float scale;
+  float softcap;             // c > 0: the scaled score becomes c tanh(score / c); 0: left as it is
   int window;                // 0: every earlier key
   int keep_first;
   const float* slopes;       // [nh] or nullptr

@@ -5,6 +5,7 @@
 //     key rows (a cached latent that serves as key and as value);
 //   * a window that also keeps the first tokens: the query at position i of its
 //     sequence sees key j <= i when i - j < window or j < keep_first;
+//   * capped scores: the scaled score s becomes c tanh(s / c);
 //   * a distance bias: slope_h * (i - j) is taken off the scaled score;
 //   * a sink: exp(sink_h) enters the softmax's denominator once, without a key
 //     or a value;
@@ -124,7 +125,9 @@ __global__ __launch_bounds__(WA_THREADS) void window_attention_kernel(const Wind
     for (int r = 0; r < KB / 16; ++r) {
       const int key = kbase + sub + 16 * r;
       const bool sees = key <= pos_c && (key >= lo_c || key < a.keep_first);
-      sc[r] = sees ? sc[r] * a.scale - slope * (float)(pos_c - key) : -INFINITY;
+      float sv = sc[r] * a.scale;
+      if (a.softcap > 0.f) sv = a.softcap * tanhf(sv / a.softcap);
+      sc[r] = sees ? sv - slope * (float)(pos_c - key) : -INFINITY;
       mx = fmaxf(mx, sc[r]);
     }
 #pragma unroll
@@ -212,7 +215,7 @@ static const char* launch_window_attention(const WindowAttention& a, dim3 grid, 
 extern "C" const char* sl_window_attention(
     const void* q, int q_stride, const void* kc, const void* vc, const int* tables, int max_pages,
     const int* cu_q, const int* positions, int num_seqs, int max_q_len, int num_tokens, int nh,
-    int nkv, int Dk, int Dv, int page, float scale, int window, int keep_first, const float* slopes,
+    int nkv, int Dk, int Dv, int page, float scale, float softcap, int window, int keep_first, const float* slopes,
     const float* sinks, const void* gate, int gate_stride, void* out, int nsplit, float* part_o,
     float* part_ml, hipStream_t stream) {
   SL_CHECK(num_seqs >= 0 && max_q_len >= 1 && nh > 0 && nkv > 0 && nh % nkv == 0,
@@ -221,7 +224,7 @@ extern "C" const char* sl_window_attention(
   SL_CHECK(vc != nullptr || Dv <= Dk, "window attention: values read from key rows cannot be wider than a key");
   SL_CHECK(page == 16 || page == 32 || page == 64, "window attention: page size must be 16, 32 or 64");
   SL_CHECK(nkv <= 65535 && num_seqs <= 65535, "window attention: grid too large");
-  SL_CHECK(window >= 0 && keep_first >= 0, "window attention: window and keep_first must be >= 0");
+  SL_CHECK(window >= 0 && keep_first >= 0 && softcap >= 0.f, "window attention: window, keep_first and the cap must be >= 0");
   SL_CHECK(nsplit >= 1 && nsplit <= 64, "window attention: 1..64 shares of the keys");
   SL_CHECK(nsplit == 1 || (part_o != nullptr && part_ml != nullptr),
            "window attention: shares of the keys need the partial buffers");
@@ -231,7 +234,7 @@ extern "C" const char* sl_window_attention(
   const long long tiles = (cols + WA_COLS - 1) / WA_COLS;
   SL_CHECK(tiles * nsplit <= 1 << 30, "window attention: too many column tiles");
   const WindowAttention a{(const act_t*)q, q_stride, (const act_t*)kc, (const act_t*)vc, tables, max_pages,
-                          cu_q, positions, nh, nkv, Dk, Dv, page, scale, window, keep_first, slopes, sinks,
+                          cu_q, positions, nh, nkv, Dk, Dv, page, scale, softcap, window, keep_first, slopes, sinks,
                           (const act_t*)gate, gate_stride, (act_t*)out, nsplit, part_o, part_ml};
   const dim3 grid((unsigned)(tiles * nsplit), nkv, num_seqs);
   const int DkP = (Dk + 3) & ~3;

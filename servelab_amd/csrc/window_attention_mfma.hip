@@ -3,7 +3,7 @@
 // SL_VK = 1: values are the first SL_DV channels of the key rows.  Same call, same meaning.
 //
 // What is float stays float.  The scores are products of bfloat16 numbers added up in float by
-// the matrix instruction (every product is exact in float); scale, distance bias, mask, the
+// the matrix instruction (every product is exact in float); scale, cap, distance bias, mask, the
 // running maximum and sum and the exponentials are float vector code.  A weight p is not rounded
 // to bfloat16 for the second product: it is cut into three bfloat16 terms p = p1 + p2 + p3 (each
 // the upper 16 bits of what the terms before left over, 8 bits of significand a term), which
@@ -130,6 +130,8 @@ __global__ __launch_bounds__(THREADS) void window_attention_mfma_kernel(const Wi
   const int pos_lo = pos0 + (wave_live ? cw0 : 0) / g, pos_hi = pos0 + (wave_live ? cw1 : 0) / g;
   const int lo_hi = a.window > 0 && pos_hi - a.window + 1 > 0 ? pos_hi - a.window + 1 : 0;
   const float scale2 = a.scale * LOG2E;
+  const bool capped = a.softcap > 0.f;
+  const float cap2 = a.softcap * LOG2E, uncap = capped ? a.scale / a.softcap : 0.f;
   const float slope2 = a.slopes != nullptr ? a.slopes[head] * LOG2E : 0.f;
   bf16x8 qf[KK];
   {
@@ -271,8 +273,11 @@ __global__ __launch_bounds__(THREADS) void window_attention_mfma_kernel(const Wi
     const float bias0 = -slope2 * (float)(pos_c - kbase - 8 * gq);
     float s[8], top = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      s[j] = fmaf(j < 4 ? s0[j] : s1[j - 4], scale2, fmaf(slope2, (float)j, bias0));
+    for (int j = 0; j < 8; ++j) {
+      const float raw = j < 4 ? s0[j] : s1[j - 4];
+      s[j] = capped ? fmaf(tanhf(raw * uncap), cap2, fmaf(slope2, (float)j, bias0))
+                    : fmaf(raw, scale2, fmaf(slope2, (float)j, bias0));
+    }
     const bool whole = kbase + 31 <= pos_lo && (kbase >= lo_hi || kbase + 31 < a.keep_first);
     if (!whole) {
 #pragma unroll
@@ -380,7 +385,7 @@ extern "C" int sl_window_attention_mfma_lds_bytes() {
 extern "C" const char* sl_window_attention_mfma(
     const void* q, int q_stride, const void* kc, const void* vc, const int* tables, int max_pages,
     const int* cu_q, const int* positions, int num_seqs, int max_q_len, int num_tokens, int nh,
-    int nkv, int Dk, int Dv, int page, float scale, int window, int keep_first, const float* slopes,
+    int nkv, int Dk, int Dv, int page, float scale, float softcap, int window, int keep_first, const float* slopes,
     const float* sinks, const void* gate, int gate_stride, void* out, int nsplit, float* part_o,
     float* part_ml, hipStream_t stream) {
   SL_CHECK(Dk == DK && Dv == DV && (vc == nullptr) == VK, "window attention (matrix cores): built for other widths");
@@ -388,7 +393,7 @@ extern "C" const char* sl_window_attention_mfma(
            "window attention: heads must be a positive multiple of kv heads");
   SL_CHECK(page == 16 || page == 32 || page == 64, "window attention: page size must be 16, 32 or 64");
   SL_CHECK(nkv <= 65535 && num_seqs <= 65535, "window attention: grid too large");
-  SL_CHECK(window >= 0 && keep_first >= 0, "window attention: window and keep_first must be >= 0");
+  SL_CHECK(window >= 0 && keep_first >= 0 && softcap >= 0.f, "window attention: window, keep_first and the cap must be >= 0");
   SL_CHECK(nsplit >= 1 && nsplit <= 64, "window attention: 1..64 shares of the keys");
   SL_CHECK(nsplit == 1 || (part_o != nullptr && part_ml != nullptr),
            "window attention: shares of the keys need the partial buffers");
@@ -398,7 +403,7 @@ extern "C" const char* sl_window_attention_mfma(
            "window attention (matrix cores): operands must be 16-byte aligned");
   if (num_seqs == 0 || num_tokens == 0) return nullptr;
   const WindowAttention a{(const act_t*)q, q_stride, (const act_t*)kc, (const act_t*)vc, tables, max_pages,
-                          cu_q, positions, nh, nkv, Dk, Dv, page, scale, window, keep_first, slopes, sinks,
+                          cu_q, positions, nh, nkv, Dk, Dv, page, scale, softcap, window, keep_first, slopes, sinks,
                           (const act_t*)gate, gate_stride, (act_t*)out, nsplit, part_o, part_ml};
   const long long cols = (long long)max_q_len * (nh / nkv);
   const long long tiles = (cols + COLS - 1) / COLS;

@@ -12,14 +12,15 @@ from .values import (KernelError, LinearWeight, PartialSums, RotationPlan, Scale
 
 class AttentionOps:
     # ----------------------------------------------------------------- rope
-    def rope_tables(self, positions, inv_freq):
+    def rope_tables(self, positions, inv_freq, magnitude=1.0):
+        """cos and sin of position x inv_freq, float32 [T, half], both times ``magnitude``."""
         T, half = positions.shape[0], inv_freq.shape[0]
         self._check(positions, torch.int32, (T,), "positions")
         self._check(inv_freq, torch.float32, (half,), "inv_freq")
         cos = self._new((T, half), torch.float32)
         sin = self._new((T, half), torch.float32)
         self._call("elementwise", "sl_rope_tables", _p(positions), _p(inv_freq), _p(cos), _p(sin),
-                   T, half)
+                   T, half, _c_float(magnitude))
         return cos, sin
 
     def _check_pages(self, k_cache, v_cache, nkv, D, page_size):

@@ -10,14 +10,35 @@ from .values import (Deferred, KernelError, PartialSums, ScaledRows, TiledRows, 
 
 class NormOps:
     # ------------------------------------------------------------ embedding
-    def embed(self, ids, table):
+    def embed(self, ids, table, scale=1.0):
+        """The rows of ``table`` at ``ids`` times ``scale``, as the float32 stream [T, H]."""
         T = ids.shape[0]
         V, H = table.shape
         self._check(ids, torch.int32, (T,), "ids")
         self._check(table, self.act_dtype, None, "embedding table")
         out = self._new((T, H), torch.float32)
-        self._call("elementwise", "sl_embed", _p(ids), _p(table), _p(out), T, H, V)
+        self._call("elementwise", "sl_embed", _p(ids), _p(table), _p(out), T, H, V, _c_float(scale))
         return out
+
+    def stream_pair(self, resid, delta, other):
+        """[resid + delta | other] as rows [T, 2 H] in the activation dtype: the float32 stream with
+        what is still to be added to it (``delta``, or None; a deferred product is run) beside a
+        second float32 stream.  Neither stream is changed."""
+        T, H = resid.shape
+        self._check(resid, torch.float32, None, "residual stream")
+        self._check(other, torch.float32, (T, H), "second stream")
+        delta = self.materialize(self._fold_deltas(resid, delta))
+        if delta is not None:
+            self._check(delta, self.act_dtype, (T, H), "delta")
+        out = self._new((T, 2 * H))
+        self._call("elementwise", "sl_stream_pair", _p(resid), _p(delta), _p(other), _p(out), T, H)
+        return out
+
+    def scale_rows(self, x, factor):
+        """x *= factor in place (float32 rows, e.g. logits)."""
+        self._check(x, torch.float32, None, "rows")
+        self._call("norm", "sl_scale", _p(x), _c_float(factor), ctypes.c_longlong(x.numel()))
+        return x
 
     # ---------------------------------------------------------------- norms
     def add_rmsnorm(self, resid, delta, weight, eps, fuse=False):
@@ -112,8 +133,8 @@ class NormOps:
 
     def gate_mul(self, gate_up, block=None, activation="silu"):
         """act(gate) * up of rows that hold gate and up interleaved in blocks of ``block`` columns
-        (default: halves); ``activation``: "silu" or "relu"."""
-        code = activation_code(activation, ("silu", "relu"))
+        (default: halves); ``activation``: "silu", "relu" or "gelu_tanh"."""
+        code = activation_code(activation, ("silu", "relu", "gelu_tanh"))
         T, two_i = gate_up.shape
         if two_i % 2:
             raise KernelError("silu_mul: the row must hold gate and up of equal width")
@@ -127,10 +148,11 @@ class NormOps:
         return out
 
     def activate(self, x, activation):
-        """act(x) in place, in float; ``activation``: "silu", "relu" or "relu2" (relu squared)."""
+        """act(x) in place, in float; ``activation``: "silu", "relu", "relu2" (relu squared) or
+        "gelu_tanh"."""
         self._check(x, self.act_dtype, None, "x")
         self._call("elementwise", "sl_activate", _p(x), _p(x), ctypes.c_longlong(x.numel()),
-                   activation_code(activation))
+                   activation_code(activation, ("silu", "relu", "relu2", "gelu_tanh")))
         return x
 
     def add_normed_rmsnorm(self, resid, y, y_weight, y_eps, weight, eps, rows=None):

@@ -375,39 +375,43 @@ class ProductOps:
 
     GATE_BLOCK = 8                # gate and up rows alternate in blocks of 8 (half an MFMA tile)
 
-    def gated_linear(self, x, weight, block, _tiled_out=False, activation="silu"):
-        """act(x Wg^T) * (x Wu^T) for a weight whose rows hold gate and up
-        interleaved in blocks of ``block`` rows (``block`` = I: plain [Wg; Wu]);
-        ``activation``: "silu" or "relu".  Few rows and a tiled weight with blocks
+    def gated_linear(self, x, weight, block, _tiled_out=False, activation="silu", bias=None):
+        """act(x Wg^T + bg) * (x Wu^T + bu) for a weight whose rows hold gate and up
+        interleaved in blocks of ``block`` rows (``block`` = I: plain [Wg; Wu]) and a
+        ``bias`` [2 I] (or None) that lies as the rows do;
+        ``activation``: "silu", "relu" or "gelu_tanh".  Few rows and a tiled weight with blocks
         of 8: one fused kernel."""
         if not isinstance(weight, LinearWeight):
             weight = LinearWeight(weight)
-        code = activation_code(activation, ("silu", "relu"))      # (what the kernels take as `gated`)
+        code = activation_code(activation, ("silu", "relu", "gelu_tanh"))      # (what the kernels take as `gated`)
+        if bias is not None:
+            self._check(bias, torch.float32, (weight.shape[0],), "bias")
         if isinstance(x, ScaledRows):
             if block != self.GATE_BLOCK or weight.shape[0] % 16:
                 raise KernelError("un-normalised rows need gate and up in blocks of 8")
-            return self._linear_scaled(x, weight, None, False, code, y_tiled=_tiled_out)
+            return self._linear_scaled(x, weight, bias, False, code, y_tiled=_tiled_out)
         M, K = x.shape
         N = weight.shape[0]
         if (_tiled_out and M < self._wide_from(K) and M <= self._few_rows_limit(weight)
                 and block == self.GATE_BLOCK and N % 16 == 0):
             self._check(x, self.act_dtype, None, "x")
             y = self._new((M, N // 2))
-            self._skinny(x, weight, None, y, M, N, K, gated=code, y_tiled=True)
+            self._skinny(x, weight, bias, y, M, N, K, gated=code, y_tiled=True)
             return TiledRows(y, (M, N // 2))
         if M <= self._few_rows_limit(weight) and block == self.GATE_BLOCK and N % 16 == 0:
             self._check(x, self.act_dtype, None, "x")
             if M >= self._wide_from(K):
                 if self._takes_mid(M, N, K):
-                    return self.linear_mid(x, weight, None, gated=code)
-                return self.linear_wide(x, weight, None, gated=code)
+                    return self.linear_mid(x, weight, bias, gated=code)
+                return self.linear_wide(x, weight, bias, gated=code)
             y = self._new((M, N // 2))
-            self._skinny(x, weight, None, y, M, N, K, gated=code)
+            self._skinny(x, weight, bias, y, M, N, K, gated=code)
             return y
-        return self.gate_mul(self.linear(x, weight, None), block, activation)
+        return self.gate_mul(self.linear(x, weight, bias), block, activation)
 
-    def gated_mlp(self, x, w_gate_up, block, w_down, defer=False, activation="silu"):
-        """down(act(gate x) * (up x)): ``gated_linear`` followed by ``linear``.  With few rows the
+    def gated_mlp(self, x, w_gate_up, block, w_down, defer=False, activation="silu", bias_gate_up=None,
+                  bias_down=None):
+        """down(act(gate x) * (up x)), with biases when given: ``gated_linear`` followed by ``linear``.  With few rows the
         kernel table keeps what lies between them in the layout its second kernel reads best
         (rows by k-step: the eight rows of a decode step then cost the down product half as many
         cache lines per load of x)."""
@@ -420,8 +424,8 @@ class ProductOps:
         tiled = (self.act_dtype == torch.bfloat16 and self.tile_few_rows and 1 < M <= self._fused_rows(w_down.shape[0])
                  and block == self.GATE_BLOCK and inner % 32 == 0 and w_gate_up.tiled is not None
                  and w_down.tiled is not None and w_down.shape[1] == inner and w_gate_up.shape[0] % 16 == 0)
-        h = self.gated_linear(x, w_gate_up, block, _tiled_out=tiled, activation=activation)
-        return self.linear(h, w_down, None, defer=defer)
+        h = self.gated_linear(x, w_gate_up, block, _tiled_out=tiled, activation=activation, bias=bias_gate_up)
+        return self.linear(h, w_down, bias_down, defer=defer)
 
     def linear_rows(self, x, w, bias, out_f32=False):
         M, K = x.shape

@@ -112,8 +112,8 @@ class RecurrentOps:
         return out
 
     def short_conv(self, buf, col, taps, state, state_off, batch, write, unit_heads=0, unit_dim=0,
-                   unit_eps=1e-6, scaled_heads=0, scale=1.0, bias=None):
-        """silu of a causal convolution over time per channel of buf[:, col:col + C] (``taps``
+                   unit_eps=1e-6, scaled_heads=0, scale=1.0, bias=None, activation="silu"):
+        """silu (``activation`` None: nothing) of a causal convolution over time per channel of buf[:, col:col + C] (``taps``
         [C, n], the last one the token's own; ``bias`` [C] is added before the silu).  The n - 1 inputs before a step come from the
         sequence's state slot at ``state_off`` ([n - 1, C], zeros at a sequence's start), and the
         step's last n - 1 inputs go back there.  The first ``unit_heads`` heads of ``unit_dim``
@@ -122,6 +122,8 @@ class RecurrentOps:
         T, stride = self._f32_rows(buf, "projected rows")
         C, n = taps.shape
         self._check(taps, torch.float32, None, "taps")
+        if activation not in (None, "silu"):
+            raise KernelError("short_conv: the activation is silu or None")
         if bias is not None:
             self._check(bias, torch.float32, (C,), "convolution bias")
         self._sequences(batch, T)
@@ -130,7 +132,7 @@ class RecurrentOps:
         self._call(self._lazy("recurrent"), "sl_short_conv", _p(buf), stride, col, C, n, _p(taps), _p(bias), _p(state),
                    _ll(slot_size), state_off, _p(batch.cu_q), _p(batch.positions), _p(batch.tok_seq),
                    _p(batch.state_slots), batch.num_seqs, T, int(bool(write)), unit_heads, unit_dim,
-                   _c_float(unit_eps), scaled_heads, _c_float(scale), _p(out))
+                   _c_float(unit_eps), scaled_heads, _c_float(scale), int(activation == "silu"), _p(out))
         return out
 
     def _scan(self, mode, src, q_col, k_col, v_col, H, G, D, Dv, log_decay, q_scale, gates, i_col, f_col,
@@ -206,12 +208,16 @@ class RecurrentOps:
 
     # ------------------------------- attention: norm over the projection, rotation, pages
     def projnorm_rope_store(self, buf, H, G, D, Dv, q_gain, k_gain, eps, rot, tables, slots, k_cache, v_cache,
-                            page_size):
+                            page_size, values_are_keys=False):
         """``buf`` (float32) holds q [H D], k [G D] and v [G Dv] side by side.  q and k are
         RMS-normed over all their heads at once (gains of that size; both None: no norm), the first ``rot`` channels of
         every head rotated in halves by ``tables``; k and v go to the token's place in the pages
-        (``slots`` None: no write); q comes back as [T, H D] in the activation dtype."""
+        (``slots`` None: no write); q comes back as [T, H D] in the activation dtype.
+        ``values_are_keys``: there is no v in ``buf``; the values cached are the keys as they lie
+        in ``buf``, before norm and rotation (Dv = D)."""
         T, stride = self._f32_rows(buf, "projected rows")
+        if values_are_keys and Dv != D:
+            raise KernelError("projnorm_rope_store: keys that serve as values have the values' width")
         if (q_gain is None) != (k_gain is None):
             raise KernelError("projnorm_rope_store: both gains or neither")
         if q_gain is not None:
@@ -231,19 +237,23 @@ class RecurrentOps:
         self._call(self._lazy("recurrent"), "sl_projnorm_rope_store", _p(buf), stride, T, H, G, D, Dv, _p(q_gain),
                    _p(k_gain), _c_float(eps), rot, _p(cos), _p(sin), _p(slots),
                    _p(k_cache) if slots is not None else None, _p(v_cache) if slots is not None else None,
-                   page_size, _p(q))
+                   page_size, _p(q), H * D if values_are_keys else (H + G) * D)
         return q
 
     # ------------------------------------------------------- routed experts
-    def route_tokens(self, logits, experts, top):
+    def route_tokens(self, logits, experts, top, over_all=False, correction=None, scale=1.0, with_matrices=None):
         """The ``top`` largest of each row's first ``experts`` logits (float32; among equals the
         lower index) with the softmax over them, and the step's (token, choice) pairs sorted by
-        expert for the grouped products."""
+        expert for the grouped products.  ``over_all``: what is compared is the softmax over all
+        ``experts`` logits plus ``correction`` [experts] (None: nothing), and a chosen expert's
+        share is its softmax value over the sum of the chosen ones' (+ 1e-20), times ``scale``.
+        ``with_matrices``: only the first so many experts have matrices (the others get no row
+        tiles; ``routed_experts`` hands their input through)."""
         T, stride = self._f32_rows(logits, "router logits")
         n = T * top
         # larger row tiles once an expert has that many rows on average: its matrices are then read
         # once per 64 or 128 rows instead of once per 16
-        per_expert = n / experts
+        per_expert = n / (experts if with_matrices is None else max(1, int(with_matrices)))
         tile_rows = _TILE_ROWS[2] if per_expert >= 2 * self.ROUTED_WIDE_TILE_ROWS else \
             (_TILE_ROWS[1] if per_expert >= self.ROUTED_WIDE_TILE_ROWS else _TILE_ROWS[0])
         max_tiles = -(-n // tile_rows) + experts
@@ -252,8 +262,12 @@ class RecurrentOps:
         order = self._new((n,), torch.int32)
         place_of = self._new((n,), torch.int32)
         tiles = self._new((max_tiles, 3), torch.int32)
+        if correction is not None:
+            self._check(correction, torch.float32, (experts,), "correction")
+        real = experts if with_matrices is None else int(with_matrices)
         self._call(self._lazy("routed"), "sl_route_tokens", _p(logits), stride, T, experts, top, _p(chosen),
-                   _p(shares), _p(order), _p(place_of), _p(tiles), max_tiles, tile_rows)
+                   _p(shares), _p(order), _p(place_of), _p(tiles), max_tiles, tile_rows, int(bool(over_all)),
+                   _p(correction), _c_float(scale), real)
         return Routing(chosen, shares, order, place_of, tiles, tile_rows)
 
     def prepare_expert_matrices(self, w, gated=False):
@@ -269,13 +283,15 @@ class RecurrentOps:
         return ExpertMatrices(tiled, w.shape, True)
 
     def routed_experts(self, x, routing, w_gate_up, w_down, base=None, activation="silu", gated=True,
-                       base_gate=None, base_gate_col=0):
+                       base_gate=None, base_gate_col=0, limit=0.0, pass_through=False):
         """sum over a token's choices of share * down_e(act(gate_e x) * up_e x), plus ``base``;
         ``w_gate_up`` [E, 2 ff, width] holds an expert's gate rows before its up rows, ``w_down``
         [E, width, ff].  ``gated`` False: an expert is down_e(act(up_e x)) and ``w_gate_up`` is
         [E, ff, width].  ``base_gate`` (float32 rows): ``base`` is multiplied by the sigmoid of
-        base_gate[t, base_gate_col].  Sums are float32; what lies between the two products is
-        rounded to the activation dtype."""
+        base_gate[t, base_gate_col].  ``activation`` "clamped_swish" (gated only): with g = min(gate_e x,
+        limit) and u = clamp(up_e x, -limit, limit) the product is g sigmoid(1.702 g) (u + 1).
+        ``pass_through``: a chosen expert beyond the E with matrices adds share * x.  Sums are
+        float32; what lies between the two products is rounded to the activation dtype."""
         code = activation_code(activation)
         if not isinstance(w_gate_up, ExpertMatrices):
             w_gate_up = ExpertMatrices(w_gate_up, w_gate_up.shape, False)
@@ -295,6 +311,8 @@ class RecurrentOps:
         top = routing.chosen.shape[1]
         n = T * top
         max_tiles = routing.tiles.shape[0]
+        if activation == "clamped_swish" and not gated:
+            raise KernelError("routed_experts: the clamped form is a gate's")
         if routing.chosen.shape[0] != T or max_tiles < -(-n // routing.tile_rows) + E:
             raise KernelError("routed_experts: the routing is for another step or other experts")
         if base is not None:
@@ -308,14 +326,15 @@ class RecurrentOps:
         mid = self._new((n, ff))
         self._call(lib, "sl_grouped_product", _p(x), _p(routing.order), top, _p(w_gate_up.data),
                    _p(routing.tiles), int(w_gate_up.tiled), max_tiles, routing.tile_rows, ff, K, int(bool(gated)), code,
-                   _p(mid))
+                   _c_float(limit), _p(mid))
         y = self._new((n, K), torch.float32)
         self._call(lib, "sl_grouped_product", _p(mid), None, 1, _p(w_down.data), _p(routing.tiles),
-                   int(w_down.tiled), max_tiles, routing.tile_rows, K, ff, 0, 0, _p(y))
+                   int(w_down.tiled), max_tiles, routing.tile_rows, K, ff, 0, 0, _c_float(0.0), _p(y))
         out = self._new((T, K))
         gate_at = None
         if base_gate is not None:
             gate_at = ctypes.c_void_p(base_gate.data_ptr() + 4 * base_gate_col)
         self._call(lib, "sl_routed_combine", _p(y), _p(routing.place_of), _p(routing.shares), T, top, _p(base),
-                   gate_at, gate_stride, K, _p(out))
+                   gate_at, gate_stride, K, _p(out), _p(routing.chosen) if pass_through else None, E,
+                   _p(x) if pass_through else None)
         return out

@@ -117,7 +117,7 @@ class ScaledRows:
 
 
 # Activations as the kernels number them (csrc/common.h).
-ACTIVATIONS = {"silu": 1, "relu": 2, "relu2": 3}
+ACTIVATIONS = {"silu": 1, "relu": 2, "relu2": 3, "gelu_tanh": 4, "clamped_swish": 5}
 
 
 def activation_code(name, allowed=None) -> int:

@@ -184,14 +184,15 @@ class WindowOps:
     # ------------------------------------------------------------ attention
     def window_attention(self, q, q_col, nh, nkv, Dk, Dv, k_cache, v_cache, page_size, block_tables,
                          batch, scale, window, keep_first=0, slopes=None, sinks=None, gate=None,
-                         gate_col=0):
+                         gate_col=0, softcap=None):
         """Attention of every token of the batch over its sequence's pages.  ``q`` [T, width]
         holds head h of a token at column ``q_col + h * Dk``; ``v_cache`` None: values are the
         first Dv channels of the key rows.  ``window`` (None: all keys) and ``keep_first``: the
         query at position i sees key j <= i when i - j < window or j < keep_first.  ``slopes``
         [nh]: slope_h * (i - j) is taken off the scaled score; ``sinks`` [nh]: exp(sink_h) joins
         the denominator; ``gate`` [T, width] with head h's gate at column ``gate_col + h``: the
-        output is multiplied by its sigmoid.  Returns [T, nh * Dv]."""
+        output is multiplied by its sigmoid.  ``softcap`` c: the scaled score s becomes
+        c tanh(s / c).  Returns [T, nh * Dv]."""
         T = q.shape[0]
         S, max_pages = block_tables.shape
         self._check(q, self.act_dtype, None, "q")
@@ -250,7 +251,8 @@ class WindowOps:
             lib, name = self._lazy("window_attention"), "sl_window_attention"
         self._call(lib, name, _c_void_p(q.data_ptr() + q_col * item), q.shape[1], _p(k_cache),
                    _p(v_cache), _p(block_tables), max_pages, _p(batch.cu_q), _p(batch.positions),
-                   S, batch.max_q_len, T, nh, nkv, Dk, Dv, page_size, _c_float(scale), window,
+                   S, batch.max_q_len, T, nh, nkv, Dk, Dv, page_size, _c_float(scale),
+                   _c_float(float(softcap or 0.0)), window,
                    int(keep_first), _p(slopes), _p(sinks),
                    _c_void_p(gate.data_ptr() + gate_col * item) if gate is not None else None, gate_stride,
                    _p(out), nsplit, _p(part_o), _p(part_ml))

@@ -1,2 +1,2 @@
 """Importing this package registers the architectures it holds."""
-from . import futezen, qwen2, topelorn, vekanex  # noqa: F401
+from . import futezen, qwen2, topelorn, vekanex, vunadra  # noqa: F401

@@ -14,7 +14,7 @@ import math
 
 import torch
 
-from .base import Mixer, PagedKVSpec, ParamSpec
+from .base import Mixer, PagedKVSpec, ParamSpec, StateSpec
 
 
 class PagedAttention(Mixer):
@@ -94,81 +94,183 @@ class PagedAttention(Mixer):
             self.w_o, None, defer=True)
 
 
+def _turning_order(rot: int, width: int, pairing: str) -> torch.Tensor:
+    """The order that puts ``width`` channels whose first ``rot`` turn in ``pairing`` pairs into
+    the order in which they turn in halves (a score does not depend on the order of its terms as
+    long as q and k agree)."""
+    if pairing == "half" or not rot:
+        return torch.arange(width)
+    return torch.cat([torch.arange(0, rot, 2), torch.arange(1, rot, 2), torch.arange(rot, width)])
+
+
 class ProjectionNormAttention(Mixer):
     """Grouped-query softmax attention whose q and k are RMS-normed over the whole projection
     (all heads of a token at once, a gain of that size) before the rotation, with biases on q,
     k, v and the output, keys of ``key_dim`` and values of ``value_dim`` channels, a score
     scale given from outside and float32 softmax weights.  The position encoding turns the
-    leading channels of a head in halves.  Causal; ``window`` None keeps every key.
+    leading channels of a head, in halves or in neighbouring pairs (the rows that make q and k
+    are then put into the order of halves at load).  Causal; ``window`` None keeps every key.
     ``projection_norm`` False: q and k go to the rotation as the projection left them (no gains
-    in the checkpoint); ``bias`` False: no biases."""
+    in the checkpoint); ``bias`` False: no biases.  ``values`` "keys": there is no value
+    projection; a token's values are its keys as the projection left them (with their bias),
+    before norm and rotation.  ``softcap`` c: a scaled score s becomes c tanh(s / c)."""
     graph_safe = True
 
     NAMES = {"q": "q", "k": "k", "v": "v", "out": "o", "q_bias": "q.b", "k_bias": "k.b",
              "v_bias": "v.b", "out_bias": "o.b", "q_norm": "q.norm", "k_norm": "k.norm"}
 
     def __init__(self, hidden_size, num_heads, num_kv_heads, key_dim, value_dim, scale, position,
-                 norm_eps, bias=True, window=None, names=None, projection_norm=True):
+                 norm_eps, bias=True, window=None, names=None, projection_norm=True, values="projected",
+                 softcap=None):
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
+        if values not in ("projected", "keys"):
+            raise ValueError("values are 'projected' or 'keys'")
         self.hidden_size = int(hidden_size)
         self.num_heads, self.num_kv_heads = int(num_heads), int(num_kv_heads)
         self.key_dim, self.value_dim = int(key_dim), int(value_dim)
+        self.values_are_keys = values == "keys"
+        if self.values_are_keys and self.value_dim != self.key_dim:
+            raise ValueError("keys that serve as values have the values' width")
         self.scale, self.norm_eps = float(scale), float(norm_eps)
         self.position = position
         self.bias = bool(bias)
         self.projection_norm = bool(projection_norm)
         self.window = None if not window else int(window)
+        self.softcap = float(softcap) if softcap else None
         self.names = dict(self.NAMES, **(names or {}))
+
+    @property
+    def in_channels(self):
+        """Channels of the input projection: q, k and (with a value projection) v."""
+        H, G, D, Dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        return (H + G) * D + (0 if self.values_are_keys else G * Dv)
 
     def param_specs(self):
         n, h = self.names, self.hidden_size
         H, G, D, Dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
-        specs = {n["q"]: ParamSpec((H * D, h)), n["k"]: ParamSpec((G * D, h)), n["v"]: ParamSpec((G * Dv, h)),
-                 n["out"]: ParamSpec((h, H * Dv))}
+        specs = {n["q"]: ParamSpec((H * D, h)), n["k"]: ParamSpec((G * D, h)), n["out"]: ParamSpec((h, H * Dv))}
+        if not self.values_are_keys:
+            specs[n["v"]] = ParamSpec((G * Dv, h))
         if self.projection_norm:
             specs.update({n["q_norm"]: ParamSpec((H * D,), init="gain"),
                           n["k_norm"]: ParamSpec((G * D,), init="gain")})
         if self.bias:
             specs.update({n["q_bias"]: ParamSpec((H * D,)), n["k_bias"]: ParamSpec((G * D,)),
-                          n["v_bias"]: ParamSpec((G * Dv,)), n["out_bias"]: ParamSpec((h,))})
+                          n["out_bias"]: ParamSpec((h,))})
+            if not self.values_are_keys:
+                specs[n["v_bias"]] = ParamSpec((G * Dv,))
         return specs
 
     def cache_spec(self):
         return PagedKVSpec(self.num_kv_heads, self.key_dim, self.window, value_dim=self.value_dim)
 
+    def _by_head(self, t, heads):
+        """Rows (or entries) of q or k, every head's channels in the order the rotation wants."""
+        by_head = t.reshape(heads, self.key_dim, *t.shape[1:])
+        return by_head[:, self.order.to(t.device)].reshape(t.shape)
+
     def load(self, tensors, rt):
         self.rt = rt
         n = self.names
+        H, G, D, Dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
         self.position.load(tensors, rt)
         layout = self.position.layout()
-        if layout is not None and (layout.pairing != "half" or layout.rot_dim > self.key_dim):
-            raise ValueError("the rotation must turn leading channels of a head in halves")
+        if layout is not None and (layout.pairing not in ("half", "interleaved") or layout.rot_dim > D):
+            raise ValueError("the rotation must turn leading channels of a head, in halves or in neighbouring pairs")
         self.rot = 0 if layout is None else int(layout.rot_dim)
-        w = torch.cat([tensors(n["q"]), tensors(n["k"]), tensors(n["v"])], 0)
+        self.order = _turning_order(self.rot, D, "half" if layout is None else layout.pairing)
+        rows = [self._by_head(tensors(n["q"]), H), self._by_head(tensors(n["k"]), G)]
+        if not self.values_are_keys:
+            rows.append(tensors(n["v"]))
+        w = torch.cat(rows, 0)
         extra = -w.shape[0] % 8
         if extra:
             w = torch.cat([w, w.new_zeros(extra, w.shape[1])], 0)
         self.w_in = rt.linear_weight(w)
         self.b_in = self.b_o = None
         if self.bias:
-            b = torch.cat([tensors(n["q_bias"]).float(), tensors(n["k_bias"]).float(),
-                           tensors(n["v_bias"]).float(), torch.zeros(extra, device=w.device)], 0)
-            self.b_in = rt.vector(b)
+            b = [self._by_head(tensors(n["q_bias"]).float(), H), self._by_head(tensors(n["k_bias"]).float(), G)]
+            if not self.values_are_keys:
+                b.append(tensors(n["v_bias"]).float())
+            self.b_in = rt.vector(torch.cat(b + [torch.zeros(extra, device=w.device)], 0))
             self.b_o = rt.vector(tensors(n["out_bias"]))
-        self.q_gain = rt.vector(tensors(n["q_norm"])) if self.projection_norm else None
-        self.k_gain = rt.vector(tensors(n["k_norm"])) if self.projection_norm else None
-        self.w_o = rt.linear_weight(tensors(n["out"]), delta=True)
+        self.q_gain = rt.vector(self._by_head(tensors(n["q_norm"]), H)) if self.projection_norm else None
+        self.k_gain = rt.vector(self._by_head(tensors(n["k_norm"]), G)) if self.projection_norm else None
+        w_o = tensors(n["out"])
+        if self.values_are_keys:
+            # the values arrive in the keys' order: the output projection's columns follow them
+            w_o = w_o.reshape(w_o.shape[0], H, Dv)[:, :, self.order.to(w_o.device)].reshape(w_o.shape)
+        self.w_o = rt.linear_weight(w_o, delta=True)
 
     def forward(self, x, batch, cache, shared):
+        buf = self.rt.ops.linear(x, self.w_in, self.b_in, out_f32=True)
+        return self._attend(buf, batch, cache, shared)
+
+    def _attend(self, buf, batch, cache, shared):
+        """``buf``: float32 rows that hold q, k and (with a value projection) v side by side."""
         ops = self.rt.ops
         H, G, D, Dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
         group = batch.groups[cache.group]
-        buf = ops.linear(x, self.w_in, self.b_in, out_f32=True)
         tables = self.position.tables(batch, shared) if self.rot else None
-        q = ops.projnorm_rope_store(buf, H, G, D, Dv, self.q_gain, self.k_gain, self.norm_eps, self.rot,
-                                    tables, group.slots if cache.write else None, cache.k, cache.v,
-                                    cache.page_size)
-        attn = ops.window_attention(q, 0, H, G, D, Dv, cache.k, cache.v, cache.page_size,
-                                    group.block_tables, batch, self.scale, self.window)
+        store = (buf, H, G, D, Dv, self.q_gain, self.k_gain, self.norm_eps, self.rot,
+                 tables, group.slots if cache.write else None, cache.k, cache.v, cache.page_size)
+        q = ops.projnorm_rope_store(*store, values_are_keys=True) if self.values_are_keys \
+            else ops.projnorm_rope_store(*store)
+        attend = (q, 0, H, G, D, Dv, cache.k, cache.v, cache.page_size, group.block_tables, batch, self.scale,
+                  self.window)
+        attn = ops.window_attention(*attend, softcap=self.softcap) if self.softcap else ops.window_attention(*attend)
         return ops.linear(attn, self.w_o, self.b_o)
+
+
+class ShortConvAttention(ProjectionNormAttention):
+    """``ProjectionNormAttention`` whose q, k and v pass a short causal convolution over time, per
+    channel and without a bias or an activation, right after the projection:
+    y_t = sum_j taps[:, j] u_(t - n + 1 + j), zeros before the sequence's start.  The last n - 1
+    projected rows of a sequence are state, so the mixer keeps pages and a state slot
+    (``cache_specs``; ``forward`` takes both bindings)."""
+
+    NAMES = dict(ProjectionNormAttention.NAMES, q_conv="q.conv", k_conv="k.conv", v_conv="v.conv")
+
+    def __init__(self, *args, conv=4, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.conv = int(conv)
+        if self.conv < 1:
+            raise ValueError("the convolution has at least one tap")
+
+    def param_specs(self):
+        specs = super().param_specs()
+        n = self.names
+        H, G, D, Dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        specs[n["q_conv"]] = ParamSpec((H * D, self.conv))
+        specs[n["k_conv"]] = ParamSpec((G * D, self.conv))
+        if not self.values_are_keys:
+            specs[n["v_conv"]] = ParamSpec((G * Dv, self.conv))
+        return specs
+
+    def cache_specs(self):
+        specs = [self.cache_spec()]
+        if self.conv > 1:
+            specs.append(StateSpec(((self.conv - 1) * self.in_channels,), "float32"))
+        return specs
+
+    def load(self, tensors, rt):
+        super().load(tensors, rt)
+        n = self.names
+        taps = [self._by_head(tensors(n["q_conv"]), self.num_heads), self._by_head(tensors(n["k_conv"]), self.num_kv_heads)]
+        if not self.values_are_keys:
+            taps.append(tensors(n["v_conv"]))
+        self.taps = rt.vector(torch.cat(taps, 0))
+        self.no_state = torch.zeros((1, 1), dtype=torch.float32, device=rt.device)
+
+    def forward(self, x, batch, caches, shared):
+        ops = self.rt.ops
+        caches = caches if isinstance(caches, (list, tuple)) else [caches]
+        pages = caches[0]
+        buf = ops.linear(x, self.w_in, self.b_in, out_f32=True)
+        if self.conv > 1:
+            state = caches[1]
+            buf = ops.short_conv(buf, 0, self.taps, state.state, 0, batch, state.write, activation=None)
+        else:                  # one tap: a factor per channel, nothing carried
+            buf = ops.short_conv(buf, 0, self.taps, self.no_state, 0, batch, False, activation=None)
+        return self._attend(buf, batch, pages, shared)

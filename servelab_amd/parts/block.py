@@ -17,6 +17,10 @@ from .base import Block, prefixed
 
 
 class PreNormBlock(Block):
+    """``feedforward`` may be None (then there is no second norm either, and the mixer's output is
+    the pending delta).  A mixer that keeps caches of several kinds declares them as a list
+    (``cache_specs``) and gets the list of bindings."""
+
     def __init__(self, norm1, mixer, norm2, feedforward,
                  names=("input_layernorm.", "self_attn.", "post_attention_layernorm.", "mlp.")):
         self.norm1, self.mixer, self.norm2, self.feedforward = norm1, mixer, norm2, feedforward
@@ -27,9 +31,13 @@ class PreNormBlock(Block):
         return all(part.graph_safe for _, part in self._children())
 
     def _children(self):
-        return list(zip(self.names, (self.norm1, self.mixer, self.norm2, self.feedforward)))
+        parts = list(zip(self.names, (self.norm1, self.mixer, self.norm2, self.feedforward)))
+        return parts if self.feedforward is not None else parts[:2]
 
     def cache_specs(self):
+        several = getattr(self.mixer, "cache_specs", None)
+        if several is not None:
+            return list(several())
         spec = self.mixer.cache_spec()
         return [] if spec is None else [spec]
 
@@ -47,9 +55,53 @@ class PreNormBlock(Block):
 
     def forward(self, resid, delta, batch, caches, shared):
         x = self.norm1.forward(resid, delta, fuse=self.mixer.takes_scaled_rows)
-        a = self.mixer.forward(x, batch, caches[0] if caches else None, shared)
+        if hasattr(self.mixer, "cache_specs"):
+            a = self.mixer.forward(x, batch, caches, shared)
+        else:
+            a = self.mixer.forward(x, batch, caches[0] if caches else None, shared)
+        if self.feedforward is None:
+            return a
         x2 = self.norm2.forward(resid, a, fuse=self.feedforward.takes_scaled_rows)
         return self.feedforward.forward(x2)
+
+
+class StreamReentry(Block):
+    """What stands before every pass over a run of layers that is walked several times: the
+    stream becomes W [x; x0] + step[t], x the stream as the layers before left it, x0 the
+    embedding output of the same tokens, W [width, 2 width] (x's columns first), step [passes,
+    width] and t = 0, 1, ... the number of the pass.  The run list calls the block once per
+    pass; which pass it is, the block counts in the step's ``shared`` dict.  It needs
+    ``ModelSpec.keeps_embedding`` and caches nothing.  The product's sums are float32 and become
+    the stream as they are."""
+    graph_safe = True
+
+    def __init__(self, hidden_size, passes, names=("in", "step")):
+        self.hidden_size, self.passes = int(hidden_size), int(passes)
+        self.names = tuple(names)
+
+    def param_specs(self):
+        from .base import ParamSpec
+        h = self.hidden_size
+        return {self.names[0]: ParamSpec((h, 2 * h)), self.names[1]: ParamSpec((self.passes, h))}
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        self.weight = rt.linear_weight(tensors(self.names[0]))
+        self.steps = rt.vector(tensors(self.names[1]))
+
+    def forward(self, resid, delta, batch, caches, shared):
+        ops = self.rt.ops
+        t = shared.get(("pass", id(self)), 0)
+        if t >= self.passes:
+            raise RuntimeError("the run list enters a repeated stretch more often than it has passes")
+        shared[("pass", id(self))] = t + 1
+        x0 = shared.get("embedding output")
+        if x0 is None:
+            raise RuntimeError("the embedding output was not kept for this step")
+        rows = ops.stream_pair(resid, delta, x0)
+        resid.copy_(ops.linear(rows, self.weight, self.steps[t], out_f32=True))
+        shared.pop("stream rows", None)
+        return None
 
 
 class ParallelBlock(Block):

@@ -44,6 +44,8 @@ class ModelSpec:
     eos_token_id: int = 0
     max_position_embeddings: int = 1 << 30
     optional_tensors: Tuple[str, ...] = ()      # names a checkpoint may hold unused
+    keeps_embedding: bool = False               # a copy of the embedding output stays at hand for
+                                                # the step's blocks (shared["embedding output"])
 
     def children(self):
         return [self.embedding] + list(self.layers) + [self.final_norm, self.head]
@@ -133,6 +135,8 @@ class DecoderModel:
         spec = self.spec
         shared: Dict[Any, Any] = {}
         resid = spec.embedding[1].forward(batch)
+        if spec.keeps_embedding:
+            shared["embedding output"] = resid.clone()
         delta = None
         for call, caches in zip(spec.run, bindings):
             delta = spec.layers[call.layer][1].forward(resid, delta, batch, caches, shared)

@@ -22,8 +22,16 @@ class EmulatedOps:
         self.act_dtype = act_dtype
 
     # ------------------------------------------------------------ embedding
-    def embed(self, ids, table):
-        return _f(table[ids.long()])
+    def embed(self, ids, table, scale=1.0):
+        return _f(table[ids.long()]) * scale
+
+    def stream_pair(self, resid, delta, other):
+        """[resid + delta | other] as rows in the activation dtype; the streams stay as they are."""
+        a = resid if delta is None else resid + _f(delta)
+        return torch.cat([a, other], -1).to(self.act_dtype)
+
+    def scale_rows(self, x, factor):
+        return x.mul_(factor)
 
     # ---------------------------------------------------------------- norms
     def add_rmsnorm(self, resid, delta, weight, eps, fuse=False):
@@ -53,6 +61,8 @@ class EmulatedOps:
     def _act(z, activation):
         if activation == "silu":
             return z * torch.sigmoid(z)
+        if activation == "gelu_tanh":
+            return 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
         return torch.relu(z) if activation == "relu" else torch.relu(z) ** 2
 
     def gate_mul(self, gate_up, block=None, activation="silu"):
@@ -83,16 +93,25 @@ class EmulatedOps:
                                     batch, scale, window)
         return self.linear(attn, w_out, bias, defer=defer)
 
-    def gated_mlp(self, x, w_gate_up, block, w_down, defer=False, activation="silu"):
-        return self.linear(self.gated_linear(x, w_gate_up, block, activation), w_down, None, defer=defer)
+    def gated_mlp(self, x, w_gate_up, block, w_down, defer=False, activation="silu", bias_gate_up=None,
+                  bias_down=None):
+        return self.linear(self.gated_linear(x, w_gate_up, block, activation, bias_gate_up), w_down, bias_down,
+                           defer=defer)
 
-    def gated_linear(self, x, w, block, activation="silu"):
-        return self.gate_mul(self.linear(x, w, None), block, activation)
+    def gated_linear(self, x, w, block, activation="silu", bias=None):
+        """(the kernels apply the gate to float32 sums; so does this)"""
+        y = _f(x) @ _f(w).T
+        if bias is not None:
+            y = y + bias
+        T, inter = y.shape[0], y.shape[1] // 2
+        gu = y.view(T, inter // block, 2, block)
+        g, u = gu[:, :, 0].reshape(T, inter), gu[:, :, 1].reshape(T, inter)
+        return (self._act(g, activation) * u).to(self.act_dtype)
 
     # ----------------------------------------------------------------- rope
-    def rope_tables(self, positions, inv_freq):
+    def rope_tables(self, positions, inv_freq, magnitude=1.0):
         ang = positions.float()[:, None] * inv_freq[None, :]
-        return torch.cos(ang), torch.sin(ang)
+        return torch.cos(ang) * magnitude, torch.sin(ang) * magnitude
 
     def rope_store(self, qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
                    pairs8=False, rot_dim=None):
@@ -229,8 +248,8 @@ class EmulatedOps:
         raise ValueError(mode)
 
     def short_conv(self, buf, col, taps, state, state_off, batch, write, unit_heads=0, unit_dim=0,
-                   unit_eps=1e-6, scaled_heads=0, scale=1.0, bias=None):
-        """silu of a causal convolution over time per channel of buf[:, col:col + C] (taps [C, n],
+                   unit_eps=1e-6, scaled_heads=0, scale=1.0, bias=None, activation="silu"):
+        """silu (``activation`` None: nothing) of a causal convolution over time per channel of buf[:, col:col + C] (taps [C, n],
         the last tap is the token's own); the n - 1 inputs before a step's first token come from
         state[slot, state_off:] laid out [n - 1, C] (oldest first; zeros at a sequence's start) and
         the step's last n - 1 inputs go back there.  The first ``unit_heads`` heads of ``unit_dim``
@@ -240,13 +259,13 @@ class EmulatedOps:
         x = buf[:, col:col + C].float()
         out = torch.empty_like(x)
         for a, b, slot, fresh in self._sequences(batch):
-            keep = state[slot, state_off:state_off + (n - 1) * C].view(n - 1, C)
+            keep = state[slot, state_off:state_off + (n - 1) * C].view(n - 1, C) if n > 1 else torch.zeros(0, C)
             past = torch.zeros(n - 1, C) if fresh else keep.clone()
             full = torch.cat([past, x[a:b]], 0)
             y = sum(full[j:j + b - a] * taps[:, j] for j in range(n))
             if bias is not None:
                 y = y + bias
-            out[a:b] = y * torch.sigmoid(y)
+            out[a:b] = y * torch.sigmoid(y) if activation == "silu" else y
             if write and n > 1:
                 keep.copy_(full[full.shape[0] - (n - 1):])
         if unit_heads:
@@ -356,7 +375,7 @@ class EmulatedOps:
 
     # -------------------------------------- attention with a norm over the projection
     def projnorm_rope_store(self, buf, H, G, D, Dv, q_gain, k_gain, eps, rot, tables, slots, k_cache,
-                            v_cache, page_size):
+                            v_cache, page_size, values_are_keys=False):
         """buf (float32) holds q [H D], k [G D], v [G Dv] side by side.  q and k are RMS-normed over
         all their heads at once, their heads' first ``rot`` channels rotated in halves; k and v go
         to the pages, q is returned [T, H D]."""
@@ -376,7 +395,8 @@ class EmulatedOps:
             return torch.cat([a * c - b * s, b * c + a * s, x[..., rot:]], -1)
         q = turned(normed(buf[:, :H * D].float(), q_gain).view(T, H, D))
         k = turned(normed(buf[:, H * D:(H + G) * D].float(), k_gain).view(T, G, D))
-        v = buf[:, (H + G) * D:(H + G) * D + G * Dv].float().view(T, G, Dv)
+        v_col = H * D if values_are_keys else (H + G) * D     # (the keys before norm and rotation)
+        v = buf[:, v_col:v_col + G * Dv].float().view(T, G, Dv)
         if slots is not None:
             page, off = (slots // page_size).long(), (slots % page_size).long()
             k_cache[page, :, off, :] = k.to(k_cache.dtype)
@@ -385,7 +405,7 @@ class EmulatedOps:
 
     def window_attention(self, q, q_col, nh, nkv, Dk, Dv, k_cache, v_cache, page_size, block_tables,
                          batch, scale, window, keep_first=0, slopes=None, sinks=None, gate=None,
-                         gate_col=0):
+                         gate_col=0, softcap=None):
         if slopes is not None or sinks is not None or gate is not None:
             raise NotImplementedError("the emulated window attention has no bias, sink or gate")
         T = q.shape[0]
@@ -410,6 +430,8 @@ class EmulatedOps:
             else:
                 v = _f(v_cache[pages, :, :, offs]).repeat_interleave(g, dim=1)
             scores = torch.einsum("qhd,rhd->hqr", qs, k) * scale
+            if softcap:
+                scores = softcap * torch.tanh(scores / softcap)
             scores = scores.masked_fill(~vis[None], float("-inf"))
             o = torch.einsum("hqr,rhd->qhd", torch.softmax(scores, -1), v)
             out[a:b] = o.reshape(b - a, nh * Dv).to(self.act_dtype)
@@ -460,15 +482,22 @@ class EmulatedOps:
             k_cache[page, 0, off, :] = row.to(k_cache.dtype)
 
     # ------------------------------------------------------- routed experts
-    def route_tokens(self, logits, experts, top):
+    def route_tokens(self, logits, experts, top, over_all=False, correction=None, scale=1.0, with_matrices=None):
         """The ``top`` largest of a row's first ``experts`` logits (float32; ties to the lower
-        index) and the softmax over them: (chosen [T, top] int32, shares [T, top] float32)."""
+        index) and the softmax over them: (chosen [T, top] int32, shares [T, top] float32).
+        ``over_all``: the largest softmax shares over all experts plus ``correction``; a chosen one's
+        share over the chosen shares' sum (+ 1e-20), times ``scale``."""
         z = logits[:, :experts].float()
+        if over_all:
+            s = torch.softmax(z, -1)
+            pick = torch.topk(s if correction is None else s + correction, top, dim=-1, sorted=True).indices
+            w = torch.gather(s, 1, pick)
+            return pick.to(torch.int32), w / (w.sum(-1, keepdim=True) + 1e-20) * scale
         best = torch.topk(z, top, dim=-1, sorted=True)
         return best.indices.to(torch.int32), torch.softmax(best.values, -1)
 
     def routed_experts(self, x, routing, w_gate_up, w_down, base=None, activation="silu", gated=True,
-                       base_gate=None, base_gate_col=0):
+                       base_gate=None, base_gate_col=0, limit=0.0, pass_through=False):
         """sum over a token's choices of share * down_e(act(gate_e x) * up_e x) (+ base);
         w_gate_up [E, 2 ff, width] holds an expert's gate rows before its up rows.  Not gated:
         down_e(act(up_e x)) with w_gate_up [E, ff, width].  base_gate: base times the sigmoid of
@@ -482,8 +511,17 @@ class EmulatedOps:
             out = out * torch.sigmoid(base_gate[:, base_gate_col].float())[:, None]
         for t in range(T):
             for e, s in zip(chosen[t].tolist(), shares[t].tolist()):
+                if e >= w_gate_up.shape[0]:         # an expert without matrices hands its input through
+                    if not pass_through:
+                        raise ValueError("an expert beyond the matrices was chosen")
+                    out[t] += s * xf[t]
+                    continue
                 gu = _f(w_gate_up[e]) @ xf[t]
-                mid = self._act(gu[:ff], activation) * gu[ff:] if gated else self._act(gu, activation)
+                if activation == "clamped_swish":
+                    g, u = gu[:ff].clamp(max=limit), gu[ff:].clamp(-limit, limit)
+                    mid = g * torch.sigmoid(1.702 * g) * (u + 1.0)
+                else:
+                    mid = self._act(gu[:ff], activation) * gu[ff:] if gated else self._act(gu, activation)
                 out[t] += s * (_f(w_down[e]) @ mid.to(self.act_dtype).float())
         return out.to(self.act_dtype)
 
