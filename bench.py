@@ -162,9 +162,41 @@ def futezen_configs(shape, layers):
     return futezen, vekanex_configs(shape, layers)[0]
 
 
+def vunadra_configs(shape, layers, window):
+    """(Vunadra config.json, Futezen config.json) of equal size: Futezen is the design nearest to it
+    (an attention over a cached latent, an attention with keys and values of their own widths through
+    the same kernels, routed experts, layers that run again).  Vunadra's layers come in the order
+    attention behind a short convolution (dense feed-forward), attention whose keys serve as values,
+    with a window and capped scores (experts), latent attention with a window (experts), attention behind a
+    convolution (experts); 64 experts and two that hand through, of which a token takes 8; with eight layers
+    or more the first two run twice."""
+    z, v, f = DESIGN_SHAPES[shape], VEKANEX_SHAPES[shape], FUTEZEN_SHAPES[shape]
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "router": {"experts": v["experts"], "identity": 2, "top": v["top"], "scale": 2.5},
+           "expert": {"ff": v["expert_ff"], "limit": 7.0}}
+    conv = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "conv": 4,
+            "scale": z["dim"] ** -0.5,
+            "rot": {"base": 5e5, "dims": z["dim"], "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}
+    keys = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "scale": z["dim"] ** -0.5,
+            "softcap": 30.0, "mask": {"size": window},
+            "rot": {"base": 5e5, "dims": z["dim"], "scaling": {"factor": 8.0, "original": 8192, "low": 1.0, "high": 4.0}}}
+    lat = {"heads": z["heads"], "dim": z["dim"], "rot_dim": f["rot_dim"], "vdim": z["dim"], "kv_rank": f["kv_rank"],
+           "scale": (z["dim"] + f["rot_dim"]) ** -0.5, "mask": {"size": window},
+           "rot": {"base": 1e6, "dims": f["rot_dim"]}}
+    order = [{"type": "attention", "mixer": conv, "mlp": dense}, {"type": "attention_2", "mixer": keys, "mlp": moe},
+             {"type": "latent_attention", "mixer": lat, "mlp": moe}, {"type": "attention", "mixer": conv, "mlp": moe}]
+    vunadra = {"architecture": "Vunadra", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-5},
+               "embedding": {"scale": 2.0}, "logit_scale": 0.5, "torch_dtype": "bfloat16",
+               "layers": [order[i % 4] for i in range(layers)]}
+    if layers >= 8:
+        vunadra["layers"] = vunadra["layers"][:layers - 2]
+        vunadra["loop"] = {"start": 0, "stop": 2, "times": 2}
+    return vunadra, futezen_configs(shape, layers)[0]
+
+
 def compare_designs(args):
     """Prefill and decode throughput of the design named by --design beside the Qwen2 decoder of equal
-    size (Futezen: beside the Vekanex decoder of equal size), at each of --design-shapes: one JSON line,
+    size (Futezen: beside the Vekanex decoder of equal size; Vunadra: beside the Futezen one), at each of --design-shapes: one JSON line,
     tokens per second each."""
     import torch
     import servelab_amd  # noqa: F401
@@ -178,8 +210,9 @@ def compare_designs(args):
                       "prefill_chunk": args.prefill_chunk, "page_size": page}, "shapes": {}}
     for shape in args.design_shapes.split(","):
         row = {}
-        other = "vekanex" if args.design == "futezen" else "qwen2"
-        pair = futezen_configs(shape, args.design_layers) if args.design == "futezen" else \
+        other = "vekanex" if args.design == "futezen" else "futezen" if args.design == "vunadra" else "qwen2"
+        pair = vunadra_configs(shape, args.design_layers, args.design_window) if args.design == "vunadra" else \
+            futezen_configs(shape, args.design_layers) if args.design == "futezen" else \
             vekanex_configs(shape, args.design_layers) if args.design == "vekanex" else \
             design_configs(shape, args.design_layers, args.design_window)
         for name, raw in zip((args.design, other), pair):
@@ -347,7 +380,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernel choice for the prompt products")
-    ap.add_argument("--design", default="", choices=["", "topelorn", "vekanex", "futezen"],
+    ap.add_argument("--design", default="", choices=["", "topelorn", "vekanex", "futezen", "vunadra"],
                     help="instead of the default workload: prefill and decode throughput of this design "
                          "beside the Qwen2 decoder of equal size")
     ap.add_argument("--design-shapes", default="3b,7b", help="comma-separated: " + ", ".join(sorted(DESIGN_SHAPES)))

@@ -179,7 +179,7 @@ LAZY_STEMS = ("window_attention", "head_gemm", "recurrent", "routed")
 # (key width, value width, values in the key rows) the matrix-core window attention is built for
 # ahead of use; other widths are compiled when a model first needs them
 WINDOW_MFMA_SIZES = ((128, 128, 0), (64, 64, 0), (576, 512, 1), (32, 16, 0), (64, 48, 1), (96, 64, 0),
-                     (96, 64, 1), (96, 80, 1), (64, 32, 1), (64, 32, 0))
+                     (96, 64, 1), (96, 80, 1), (64, 32, 1), (64, 32, 0), (96, 96, 0), (32, 48, 0))
 
 
 def all_units(head_dims=(32, 64, 96, 128, 192, 256)) -> List[Unit]:
