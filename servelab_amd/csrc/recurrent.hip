@@ -579,15 +579,41 @@ extern "C" const char* sl_head_norm_gate(const float* o, int T, int H, int Dv, c
 // in the activation type; k and v go to the token's place in the pages.  The values lie at column
 // v_col of the row (behind k: (H + G) D; at H D the values are the keys as the projection left
 // them, before norm and rotation).  One block per token.
+// With taps given, the row's first conv_C channels first pass a short causal convolution over time
+// (no bias, no activation; the sums of short_conv_kernel in the same order): the block leaves its
+// token's sums in LDS and goes on from there, so the convolved rows never reach memory.  The
+// state's new last inputs are written by short_conv_state_kernel, launched behind this one.
 __global__ void projnorm_rope_store_kernel(const float* __restrict__ buf, int stride, int H, int G, int D, int Dv,
                                            const float* __restrict__ qw, const float* __restrict__ kw, float eps,
                                            int rot, const float* __restrict__ cosv, const float* __restrict__ sinv,
                                            const int* __restrict__ slots, act_t* __restrict__ kc,
                                            act_t* __restrict__ vc, int page, act_t* __restrict__ q_out,
-                                           int v_col) {
+                                           int v_col, const ShortConv cv) {
   __shared__ float scratch[16];
+  extern __shared__ float convolved[];       // [cv.C] when a convolution comes first
   const size_t t = blockIdx.x;
   const float* row = buf + t * stride;
+  if (cv.w != nullptr) {
+    const int s = cv.tok_seq[t];
+    const int first = cv.cu_q[s];
+    const int i = (int)t - first;
+    const bool fresh = cv.positions[first] == 0;
+    const float* past = cv.state + (size_t)cv.slots[s] * cv.state_stride + cv.state_off;
+    const int back = cv.taps - 1;
+    for (int c = threadIdx.x; c < cv.C; c += blockDim.x) {
+      float acc = 0.f;
+      for (int j = 0; j < cv.taps; ++j) {
+        const int idx = i - back + j;
+        float x;
+        if (idx >= 0) x = buf[(size_t)(first + idx) * stride + c];
+        else x = fresh ? 0.f : past[(size_t)(back + idx) * cv.C + c];
+        acc += cv.w[(size_t)c * cv.taps + j] * x;
+      }
+      convolved[c] = acc;
+    }
+    __syncthreads();
+    row = convolved;
+  }
   const int nq = H * D, nk = G * D, nv = G * Dv;
   float sq = 0.f, sk = 0.f;
   const bool normed = qw != nullptr;
@@ -625,10 +651,76 @@ __global__ void projnorm_rope_store_kernel(const float* __restrict__ buf, int st
       vc[((pg * G + e / Dv) * Dv + e % Dv) * page + off] = from_f<act_t>(row[v_col + e]);
 }
 
+// The same without a norm over the projection, where nothing ties a token's heads together: one
+// wavefront per (token, head of q, k or v), so that a step of few tokens still fills the chip
+// and the convolution's loads (a head's channels over the taps, and their partners' for the
+// rotation) are all in flight together.  The sums run in the order of the kernel above.
+__global__ __launch_bounds__(64) void rope_store_heads_kernel(const float* __restrict__ buf, int stride, int H, int G, int D,
+                                                              int Dv, int rot, const float* __restrict__ cosv,
+                                                              const float* __restrict__ sinv,
+                                                              const int* __restrict__ slots, act_t* __restrict__ kc,
+                                                              act_t* __restrict__ vc, int page,
+                                                              act_t* __restrict__ q_out, int v_col, const ShortConv cv) {
+  const size_t t = blockIdx.x;
+  const int hb = blockIdx.y, lane = threadIdx.x;
+  const float* row = buf + t * stride;
+  int first = 0, i = 0, back = 0;
+  bool fresh = true;
+  const float* past = nullptr;
+  if (cv.w != nullptr) {
+    const int s = cv.tok_seq[t];
+    first = cv.cu_q[s];
+    i = (int)t - first;
+    fresh = cv.positions[first] == 0;
+    past = cv.state + (size_t)cv.slots[s] * cv.state_stride + cv.state_off;
+    back = cv.taps - 1;
+  }
+  auto value = [&](int c) -> float {
+    if (cv.w == nullptr) return row[c];
+    float acc = 0.f;
+    for (int j = 0; j < cv.taps; ++j) {
+      const int idx = i - back + j;
+      float x;
+      if (idx >= 0) x = buf[(size_t)(first + idx) * stride + c];
+      else x = fresh ? 0.f : past[(size_t)(back + idx) * cv.C + c];
+      acc += cv.w[(size_t)c * cv.taps + j] * x;
+    }
+    return acc;
+  };
+  const int slot = slots != nullptr ? slots[t] : 0;
+  const size_t pg = slot / page, off = slot % page;
+  if (hb >= H + G) {                                   // a head of v
+    if (slots == nullptr) return;
+    const int g = hb - H - G;
+    for (int d = lane; d < Dv; d += 64)
+      vc[((pg * G + g) * Dv + d) * page + off] = from_f<act_t>(value(v_col + g * Dv + d));
+    return;
+  }
+  const bool is_q = hb < H;
+  if (!is_q && slots == nullptr) return;
+  const int base = hb * D;                             // (k heads follow the q heads in the row)
+  const int half = rot / 2;
+  for (int d = lane; d < D; d += 64) {
+    float v = value(base + d);
+    if (d < rot) {
+      const int p = d < half ? d : d - half;
+      const float o = value(base + (d < half ? d + half : d - half));
+      const float cs = cosv[t * half + p], sn = sinv[t * half + p];
+      v = d < half ? v * cs - o * sn : v * cs + o * sn;
+    }
+    if (is_q) q_out[t * (size_t)(H * D) + base + d] = from_f<act_t>(v);
+    else kc[((pg * G + (hb - H)) * page + off) * D + d] = from_f<act_t>(v);
+  }
+}
+
 extern "C" const char* sl_projnorm_rope_store(const float* buf, int stride, int T, int H, int G, int D, int Dv,
                                               const float* qw, const float* kw, float eps, int rot,
                                               const float* cosv, const float* sinv, const int* slots, void* kc,
-                                              void* vc, int page, void* q_out, int v_col, hipStream_t stream) {
+                                              void* vc, int page, void* q_out, int v_col,
+                                              const float* taps_w, int taps, int conv_C, float* state,
+                                              long long state_stride, int state_off, const int* cu_q,
+                                              const int* positions, const int* tok_seq, const int* state_slots,
+                                              int S, int write_state, hipStream_t stream) {
   SL_CHECK(T >= 0 && H > 0 && G > 0 && D > 0 && Dv > 0 && page > 0, "projnorm_rope_store: sizes must be positive");
   SL_CHECK((long long)(H + G) * D <= stride && v_col >= 0 && v_col + (long long)G * Dv <= stride,
            "projnorm_rope_store: q, k and v do not fit the rows");
@@ -636,8 +728,31 @@ extern "C" const char* sl_projnorm_rope_store(const float* buf, int stride, int 
   SL_CHECK(rot == 0 || (cosv != nullptr && sinv != nullptr), "projnorm_rope_store: cos and sin are missing");
   SL_CHECK((qw == nullptr) == (kw == nullptr), "projnorm_rope_store: both gains or neither");
   SL_CHECK(slots == nullptr || (kc != nullptr && vc != nullptr), "projnorm_rope_store: pages are missing");
+  ShortConv cv{};
+  size_t lds = 0;
+  if (taps_w != nullptr) {
+    SL_CHECK(taps >= 1 && taps <= 64 && conv_C > 0 && conv_C <= stride && conv_C <= 12288,
+             "projnorm_rope_store: a convolution of 1..64 taps over at most 12,288 channels within the rows");
+    SL_CHECK(v_col + (long long)G * Dv <= conv_C, "projnorm_rope_store: q, k and v must all pass the convolution");
+    SL_CHECK(cu_q != nullptr && positions != nullptr && tok_seq != nullptr && state_slots != nullptr && state != nullptr,
+             "projnorm_rope_store: the convolution needs the step's sequences and a state");
+    SL_CHECK(state_off >= 0 && state_off + (long long)(taps - 1) * conv_C <= state_stride,
+             "projnorm_rope_store: the last inputs do not fit the state slot");
+    cv = ShortConv{buf, stride, 0, conv_C, taps, taps_w, nullptr, state, state_stride, state_off, cu_q, positions,
+                   tok_seq, state_slots, 0, 0, 0, 0.f, 1.f, 0, nullptr};
+    lds = (size_t)conv_C * sizeof(float);
+  }
   if (T == 0) return nullptr;
-  projnorm_rope_store_kernel<<<T, 256, 0, stream>>>(buf, stride, H, G, D, Dv, qw, kw, eps, rot, cosv, sinv, slots,
-                                                    (act_t*)kc, (act_t*)vc, page, (act_t*)q_out, v_col);
+  // (few tokens: a wavefront per head fills the chip; many: a block per token computes every channel's
+  // convolution once, where the heads' wavefronts compute the rotated ones twice: 2,048 tokens of 20 heads
+  // of 128 channels, 4 taps: 32 against 50 us; 8 tokens: 28 against 9 us)
+  if (qw == nullptr && H + 2 * G <= 65535 && T < 512)
+    rope_store_heads_kernel<<<dim3(T, H + 2 * G), 64, 0, stream>>>(buf, stride, H, G, D, Dv, rot, cosv, sinv, slots,
+                                                                   (act_t*)kc, (act_t*)vc, page, (act_t*)q_out, v_col, cv);
+  else
+    projnorm_rope_store_kernel<<<T, 256, lds, stream>>>(buf, stride, H, G, D, Dv, qw, kw, eps, rot, cosv, sinv, slots,
+                                                        (act_t*)kc, (act_t*)vc, page, (act_t*)q_out, v_col, cv);
+  if (taps_w != nullptr && write_state && taps > 1)
+    short_conv_state_kernel<<<dim3(S, (conv_C + 255) / 256), 256, 0, stream>>>(cv, S);
   return sl_launch_status();
 }

@@ -44,12 +44,26 @@ __global__ __launch_bounds__(64) void route_kernel(const float* __restrict__ log
   unsigned long long taken = 0ull;             // bit u: element lane + 64 u is chosen already (E <= 4096)
   float mine = 0.f;                            // lane k keeps the k-th largest logit
   int mine_e = 0;
+  auto number = [&](int e) -> float {          // what the experts are compared by
+    const float v = z[e];
+    return over_all ? expf(v - zmax) * inv_sum + (correction != nullptr ? correction[e] : 0.f) : v;
+  };
+  float kept[4];                               // a lane's first four numbers stay in registers (E <= 256: all)
+#pragma unroll
+  for (int u = 0; u < 4; ++u) kept[u] = lane + 64 * u < E ? number(lane + 64 * u) : -INFINITY;
   for (int k = 0; k < top; ++k) {
     float best = -INFINITY;
     int at = 0x7fffffff;
-    for (int u = 0, e = lane; e < E; ++u, e += 64) {
-      float v = z[e];
-      if (over_all) v = expf(v - zmax) * inv_sum + (correction != nullptr ? correction[e] : 0.f);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = lane + 64 * u;
+      if (e < E && !((taken >> u) & 1ull) && (kept[u] > best || (kept[u] == best && e < at))) {
+        best = kept[u];
+        at = e;
+      }
+    }
+    for (int u = 4, e = lane + 256; e < E; ++u, e += 64) {
+      const float v = number(e);
       if (!((taken >> u) & 1ull) && (v > best || (v == best && e < at))) {
         best = v;
         at = e;

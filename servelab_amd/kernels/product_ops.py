@@ -407,7 +407,10 @@ class ProductOps:
             y = self._new((M, N // 2))
             self._skinny(x, weight, bias, y, M, N, K, gated=code)
             return y
-        return self.gate_mul(self.linear(x, weight, bias), block, activation)
+        if bias is not None:
+            # (the gate sees float32 sums with their bias, as in the fused kernels' epilogues)
+            return self.gate_mul_sums(self.linear(x, weight, None, out_f32=True), bias, block, activation)
+        return self.gate_mul(self.linear(x, weight, None), block, activation)
 
     def gated_mlp(self, x, w_gate_up, block, w_down, defer=False, activation="silu", bias_gate_up=None,
                   bias_down=None):

@@ -207,15 +207,24 @@ class RecurrentOps:
         return out
 
     # ------------------------------- attention: norm over the projection, rotation, pages
+    CONV_IN_STORE_MAX_CHANNELS = 12288    # (a token's convolved row waits in 48 KB of LDS)
+
     def projnorm_rope_store(self, buf, H, G, D, Dv, q_gain, k_gain, eps, rot, tables, slots, k_cache, v_cache,
-                            page_size, values_are_keys=False):
+                            page_size, values_are_keys=False, conv=None):
         """``buf`` (float32) holds q [H D], k [G D] and v [G Dv] side by side.  q and k are
         RMS-normed over all their heads at once (gains of that size; both None: no norm), the first ``rot`` channels of
         every head rotated in halves by ``tables``; k and v go to the token's place in the pages
         (``slots`` None: no write); q comes back as [T, H D] in the activation dtype.
         ``values_are_keys``: there is no v in ``buf``; the values cached are the keys as they lie
-        in ``buf``, before norm and rotation (Dv = D)."""
+        in ``buf``, before norm and rotation (Dv = D).  ``conv`` = (taps [C, n], state, state_off, batch,
+        write): q, k and v (the row's first C channels) first pass the short causal convolution of
+        ``short_conv`` without bias and activation, in the same launch; the state's last inputs are
+        renewed when ``write``."""
         T, stride = self._f32_rows(buf, "projected rows")
+        if conv is not None and conv[0].shape[0] > self.CONV_IN_STORE_MAX_CHANNELS:
+            taps, state, state_off, batch, write = conv
+            buf = self.short_conv(buf, 0, taps, state, state_off, batch, write, activation=None)
+            stride, conv = buf.shape[1], None
         if values_are_keys and Dv != D:
             raise KernelError("projnorm_rope_store: keys that serve as values have the values' width")
         if (q_gain is None) != (k_gain is None):
@@ -237,8 +246,22 @@ class RecurrentOps:
         self._call(self._lazy("recurrent"), "sl_projnorm_rope_store", _p(buf), stride, T, H, G, D, Dv, _p(q_gain),
                    _p(k_gain), _c_float(eps), rot, _p(cos), _p(sin), _p(slots),
                    _p(k_cache) if slots is not None else None, _p(v_cache) if slots is not None else None,
-                   page_size, _p(q), H * D if values_are_keys else (H + G) * D)
+                   page_size, _p(q), H * D if values_are_keys else (H + G) * D, *self._conv_args(conv, T, stride))
         return q
+
+    def _conv_args(self, conv, T, stride):
+        """The convolution's part of ``sl_projnorm_rope_store``'s arguments."""
+        if conv is None:
+            return (None, 0, 0, None, _ll(0), 0, None, None, None, None, 0, 0)
+        taps, state, state_off, batch, write = conv
+        C, n = taps.shape
+        self._check(taps, torch.float32, None, "taps")
+        self._sequences(batch, T)
+        slot_size = self._state(state, state_off + (n - 1) * C)
+        if C > stride:
+            raise KernelError("projnorm_rope_store: the convolution's channels do not fit the rows")
+        return (_p(taps), n, C, _p(state), _ll(slot_size), state_off, _p(batch.cu_q), _p(batch.positions),
+                _p(batch.tok_seq), _p(batch.state_slots), batch.num_seqs, int(bool(write)))
 
     # ------------------------------------------------------- routed experts
     def route_tokens(self, logits, experts, top, over_all=False, correction=None, scale=1.0, with_matrices=None):

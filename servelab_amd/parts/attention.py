@@ -207,16 +207,21 @@ class ProjectionNormAttention(Mixer):
         buf = self.rt.ops.linear(x, self.w_in, self.b_in, out_f32=True)
         return self._attend(buf, batch, cache, shared)
 
-    def _attend(self, buf, batch, cache, shared):
-        """``buf``: float32 rows that hold q, k and (with a value projection) v side by side."""
+    def _attend(self, buf, batch, cache, shared, conv=None):
+        """``buf``: float32 rows that hold q, k and (with a value projection) v side by side;
+        ``conv``: a short convolution they pass first, in the launch that norms, turns and stores."""
         ops = self.rt.ops
         H, G, D, Dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
         group = batch.groups[cache.group]
         tables = self.position.tables(batch, shared) if self.rot else None
         store = (buf, H, G, D, Dv, self.q_gain, self.k_gain, self.norm_eps, self.rot,
                  tables, group.slots if cache.write else None, cache.k, cache.v, cache.page_size)
-        q = ops.projnorm_rope_store(*store, values_are_keys=True) if self.values_are_keys \
-            else ops.projnorm_rope_store(*store)
+        more = {}
+        if self.values_are_keys:
+            more["values_are_keys"] = True
+        if conv is not None:
+            more["conv"] = conv
+        q = ops.projnorm_rope_store(*store, **more)
         attend = (q, 0, H, G, D, Dv, cache.k, cache.v, cache.page_size, group.block_tables, batch, self.scale,
                   self.window)
         attn = ops.window_attention(*attend, softcap=self.softcap) if self.softcap else ops.window_attention(*attend)
@@ -270,7 +275,7 @@ class ShortConvAttention(ProjectionNormAttention):
         buf = ops.linear(x, self.w_in, self.b_in, out_f32=True)
         if self.conv > 1:
             state = caches[1]
-            buf = ops.short_conv(buf, 0, self.taps, state.state, 0, batch, state.write, activation=None)
+            conv = (self.taps, state.state, 0, batch, state.write)
         else:                  # one tap: a factor per channel, nothing carried
-            buf = ops.short_conv(buf, 0, self.taps, self.no_state, 0, batch, False, activation=None)
-        return self._attend(buf, batch, pages, shared)
+            conv = (self.taps, self.no_state, 0, batch, False)
+        return self._attend(buf, batch, pages, shared, conv=conv)

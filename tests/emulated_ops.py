@@ -73,6 +73,13 @@ class EmulatedOps:
         g, u = gu[:, :, 0].reshape(T, inter), gu[:, :, 1].reshape(T, inter)
         return (self._act(g, activation) * u).to(self.act_dtype)
 
+    def gate_mul_sums(self, sums, bias, block=None, activation="silu"):
+        y = sums if bias is None else sums + bias
+        T, inter = y.shape[0], y.shape[1] // 2
+        block = inter if block is None else block
+        gu = y.view(T, inter // block, 2, block)
+        return (self._act(gu[:, :, 0].reshape(T, inter), activation) * gu[:, :, 1].reshape(T, inter)).to(self.act_dtype)
+
     def activate(self, x, activation):
         return x.copy_(self._act(_f(x), activation).to(x.dtype))
 
@@ -375,11 +382,14 @@ class EmulatedOps:
 
     # -------------------------------------- attention with a norm over the projection
     def projnorm_rope_store(self, buf, H, G, D, Dv, q_gain, k_gain, eps, rot, tables, slots, k_cache,
-                            v_cache, page_size, values_are_keys=False):
+                            v_cache, page_size, values_are_keys=False, conv=None):
         """buf (float32) holds q [H D], k [G D], v [G Dv] side by side.  q and k are RMS-normed over
         all their heads at once, their heads' first ``rot`` channels rotated in halves; k and v go
         to the pages, q is returned [T, H D]."""
         T = buf.shape[0]
+        if conv is not None:        # q, k and v first pass a short convolution without an activation
+            taps, state, state_off, batch, write = conv
+            buf = self.short_conv(buf, 0, taps, state, state_off, batch, write, activation=None)
 
         def normed(x, gain):
             if gain is None:        # no norm over the projection

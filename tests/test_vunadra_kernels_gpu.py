@@ -61,6 +61,11 @@ def test_gelu_gate_and_activation(dtype):
         gu = (2 * torch.randn(T, 2 * inter, generator=g)).to(dtype)
         close(hip.gate_mul(gu.to(DEV), block, "gelu_tanh"), emu.gate_mul(gu, block, "gelu_tanh"), tol)
         close(hip.activate(gu.clone().to(DEV), "gelu_tanh"), emu.activate(gu.clone(), "gelu_tanh"), tol)
+    for T, inter, block in ((3, 40, 8), (17, 96, None), (130, 24, 8), (2, 10, 5)):
+        sums, bias = 2 * torch.randn(T, 2 * inter, generator=g), torch.randn(2 * inter, generator=g)
+        for b in (bias, None):
+            close(hip.gate_mul_sums(sums.to(DEV), None if b is None else b.to(DEV), block, "gelu_tanh"),
+                  emu.gate_mul_sums(sums, b, block, "gelu_tanh"), tol)
     z = torch.linspace(-6, 6, 25, dtype=torch.float64)
     want = 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
     close(emu.activate(z.float().clone(), "gelu_tanh"), want, 1e-6)
@@ -241,3 +246,46 @@ def test_experts_routed_by_shares_with_a_correction(dtype, experts, through, top
     loose = emu.routed_experts(x, (chosen, shares), w_gu, w_d, None, activation="clamped_swish", gated=True, limit=50.0,
                                pass_through=through > 0)
     assert (loose.float() - want.float()).abs().max() > 0.05                  # (the clamps matter)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("taps", [1, 3, 4])
+def test_convolution_inside_the_launch_that_turns_and_stores(dtype, taps):
+    """q, k and v pass the convolution in the launch that norms, turns and stores them: the same rows,
+    pages and last inputs as the two calls one after the other."""
+    hip, emu = tables(dtype)
+    g = torch.Generator().manual_seed(7 + taps)
+    T = sum(Q_LENS)
+    batch_d, batch_h = fake_batch(Q_LENS, STARTS, SLOTS, DEV), fake_batch(Q_LENS, STARTS, SLOTS, "cpu")
+    for H, G, D, Dv, rot, normed in ((4, 2, 16, 24, 16, False), (3, 3, 10, 6, 4, True), (6, 3, 64, 32, 64, False)):
+        C = (H + G) * D + G * Dv
+        buf = torch.randn(T, C + 5, generator=g)
+        w = 0.6 * torch.randn(C, taps, generator=g)
+        qg = 1 + 0.3 * torch.randn(H * D, generator=g) if normed else None
+        kg = 1 + 0.3 * torch.randn(G * D, generator=g) if normed else None
+        ang = torch.rand(T, rot // 2, generator=g) * 6
+        tb = RotaryTables(torch.cos(ang), torch.sin(ang))
+        tbd = RotaryTables(tb.cos.to(DEV), tb.sin.to(DEV))
+        page = 16
+        slots = torch.randperm(8 * page, generator=g)[:T].to(torch.int32)
+        kc2, vc2 = torch.zeros(8, G, page, D).to(dtype), torch.zeros(8, G, Dv, page).to(dtype)
+        kd, vd = kc2.clone().to(DEV), vc2.clone().to(DEV)
+        st = states(6, max(1, (taps - 1) * C) + 2, seed=8)
+        s1, s2 = st.clone().to(DEV), st.clone()
+        dev = lambda t: None if t is None else t.to(DEV)
+        q1 = hip.projnorm_rope_store(buf.to(DEV), H, G, D, Dv, dev(qg), dev(kg), 1e-5, rot, tbd, slots.to(DEV), kd, vd,
+                                     page, conv=(w.to(DEV), s1, 0, batch_d, True))
+        q2 = emu.projnorm_rope_store(buf, H, G, D, Dv, qg, kg, 1e-5, rot, tb, slots, kc2, vc2, page,
+                                     conv=(w, s2, 0, batch_h, True))
+        tol = 3e-6 if dtype == torch.float32 else 8e-3
+        close(q1, q2, tol)
+        close(kd, kc2, tol)
+        close(vd, vc2, tol)
+        if taps > 1:
+            close(s1[sorted(SLOTS)][:, :(taps - 1) * C], s2[sorted(SLOTS)][:, :(taps - 1) * C], 0)
+        # and the two calls one after the other on the device give the same bits
+        s3 = st.clone().to(DEV)
+        k3, v3 = torch.zeros_like(kd), torch.zeros_like(vd)
+        rows = hip.short_conv(buf.to(DEV), 0, w.to(DEV), s3, 0, batch_d, True, activation=None)
+        q3 = hip.projnorm_rope_store(rows, H, G, D, Dv, dev(qg), dev(kg), 1e-5, rot, tbd, slots.to(DEV), k3, v3, page)
+        assert torch.equal(q1, q3) and torch.equal(kd, k3) and torch.equal(vd, v3)
