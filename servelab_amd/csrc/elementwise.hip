@@ -135,34 +135,6 @@ extern "C" const char* sl_gate_mul(const void* gate_up, void* out, int T, int I,
   return sl_launch_status();
 }
 
-// The same from the float sums of the gate/up product and its bias (which lies as the columns do):
-// out[t, i] = act(sum_gate + bias_gate) * (sum_up + bias_up), rounded once.
-__global__ void gate_mul_sums_kernel(const float* __restrict__ sums, const float* __restrict__ bias,
-                                     act_t* __restrict__ out, int I, int block, size_t total, int act) {
-  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-       idx += (size_t)gridDim.x * blockDim.x) {
-    const size_t t = idx / I;
-    const int i = (int)(idx - t * I);
-    const int col = 2 * block * (i / block) + i % block;
-    const size_t at = t * 2 * I + col;
-    const float g = sums[at] + (bias != nullptr ? bias[col] : 0.f);
-    const float u = sums[at + block] + (bias != nullptr ? bias[col + block] : 0.f);
-    out[idx] = from_f<act_t>(sl_act(g, act) * u);
-  }
-}
-
-extern "C" const char* sl_gate_mul_sums(const float* sums, const float* bias, void* out, int T, int I, int block,
-                                        int act, hipStream_t stream) {
-  SL_CHECK(T >= 0 && I > 0, "gate_mul_sums: sizes must be positive");
-  SL_CHECK(act >= SL_ACT_SILU && act <= SL_ACT_GELU_TANH, "gate_mul_sums: unknown activation");
-  SL_CHECK(block > 0 && I % block == 0, "gate_mul_sums: the block must divide the width");
-  if (T == 0) return nullptr;
-  const size_t total = (size_t)T * I;
-  const int blocks = (int)((total + 255) / 256 < 65535 * 4 ? (total + 255) / 256 : 65535 * 4);
-  gate_mul_sums_kernel<<<blocks, 256, 0, stream>>>(sums, bias, (act_t*)out, I, block, total, act);
-  return sl_launch_status();
-}
-
 extern "C" const char* sl_silu_mul(const void* gate_up, void* out, int T, int I, int block,
                                    hipStream_t stream) {
   return sl_gate_mul(gate_up, out, T, I, block, SL_ACT_SILU, stream);

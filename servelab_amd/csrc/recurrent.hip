@@ -749,8 +749,8 @@ extern "C" const char* sl_projnorm_rope_store(const float* buf, int stride, int 
   if (qw == nullptr && H + 2 * G <= 65535 && T < 512)
     rope_store_heads_kernel<<<dim3(T, H + 2 * G), 64, 0, stream>>>(buf, stride, H, G, D, Dv, rot, cosv, sinv, slots,
                                                                    (act_t*)kc, (act_t*)vc, page, (act_t*)q_out, v_col, cv);
-  else
-    projnorm_rope_store_kernel<<<T, 256, lds, stream>>>(buf, stride, H, G, D, Dv, qw, kw, eps, rot, cosv, sinv, slots,
+  else   // (a step of few tokens has few blocks: wider ones shorten each block's loops over the row)
+    projnorm_rope_store_kernel<<<T, T <= 64 ? 1024 : 256, lds, stream>>>(buf, stride, H, G, D, Dv, qw, kw, eps, rot, cosv, sinv, slots,
                                                         (act_t*)kc, (act_t*)vc, page, (act_t*)q_out, v_col, cv);
   if (taps_w != nullptr && write_state && taps > 1)
     short_conv_state_kernel<<<dim3(S, (conv_C + 255) / 256), 256, 0, stream>>>(cv, S);

@@ -147,22 +147,6 @@ class NormOps:
         self._call("elementwise", "sl_gate_mul", _p(gate_up), _p(out), T, inter, block, code)
         return out
 
-    def gate_mul_sums(self, sums, bias, block=None, activation="silu"):
-        """``gate_mul`` from the float32 sums of the gate/up product and its ``bias`` [2 I] (or None),
-        which lies as the columns do: act(gate + b) * (up + b) with one rounding."""
-        code = activation_code(activation, ("silu", "relu", "relu2", "gelu_tanh"))
-        T, two_i = sums.shape
-        inter = two_i // 2
-        block = inter if block is None else int(block)
-        if two_i % 2 or block < 1 or inter % block:
-            raise KernelError("gate_mul_sums: the row must hold gate and up in blocks that divide their width")
-        self._check(sums, torch.float32, None, "gate/up sums")
-        if bias is not None:
-            self._check(bias, torch.float32, (two_i,), "bias")
-        out = self._new((T, inter))
-        self._call("elementwise", "sl_gate_mul_sums", _p(sums), _p(bias), _p(out), T, inter, block, code)
-        return out
-
     def activate(self, x, activation):
         """act(x) in place, in float; ``activation``: "silu", "relu", "relu2" (relu squared) or
         "gelu_tanh"."""

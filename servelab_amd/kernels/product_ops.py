@@ -407,10 +407,7 @@ class ProductOps:
             y = self._new((M, N // 2))
             self._skinny(x, weight, bias, y, M, N, K, gated=code)
             return y
-        if bias is not None:
-            # (the gate sees float32 sums with their bias, as in the fused kernels' epilogues)
-            return self.gate_mul_sums(self.linear(x, weight, None, out_f32=True), bias, block, activation)
-        return self.gate_mul(self.linear(x, weight, None), block, activation)
+        return self.gate_mul(self.linear(x, weight, bias), block, activation)
 
     def gated_mlp(self, x, w_gate_up, block, w_down, defer=False, activation="silu", bias_gate_up=None,
                   bias_down=None):
@@ -491,7 +488,26 @@ class ProductOps:
         that a row gives the same values whichever path its step takes."""
         if bias is None:
             return self.library_sums(x, w)
+        b16 = self._bias_as_bfloat16(bias)
+        if b16 is not None:
+            # a bias that bfloat16 holds exactly (one that a bfloat16 checkpoint stored): the library adds it
+            # to its float32 sums in the product's epilogue, before the one rounding
+            M = x.shape[0]
+            rows = self.library_rows(M)
+            if rows != M:
+                padded = self._new((rows, x.shape[1]))
+                padded[:M].copy_(x)
+                x = padded
+            return torch.addmm(b16, x, w.t())[:M]
         return self.library_sums(x, w, torch.float32).add_(bias).to(torch.bfloat16)
+
+    def _bias_as_bfloat16(self, bias):
+        """``bias`` in bfloat16 when that loses nothing, else None; looked at once per bias (the first many-row
+        product that adds it, which no captured step contains)."""
+        if not hasattr(bias, "_as_bfloat16"):         # (kept on the tensor itself: it lives as long as the bias)
+            b16 = bias.to(torch.bfloat16)
+            bias._as_bfloat16 = b16 if bool(torch.equal(b16.float(), bias)) else None
+        return bias._as_bfloat16
 
     @contextlib.contextmanager
     def library_tuning(self, max_ms: int = 30, results_file: Optional[str] = None):

@@ -73,13 +73,6 @@ class EmulatedOps:
         g, u = gu[:, :, 0].reshape(T, inter), gu[:, :, 1].reshape(T, inter)
         return (self._act(g, activation) * u).to(self.act_dtype)
 
-    def gate_mul_sums(self, sums, bias, block=None, activation="silu"):
-        y = sums if bias is None else sums + bias
-        T, inter = y.shape[0], y.shape[1] // 2
-        block = inter if block is None else block
-        gu = y.view(T, inter // block, 2, block)
-        return (self._act(gu[:, :, 0].reshape(T, inter), activation) * gu[:, :, 1].reshape(T, inter)).to(self.act_dtype)
-
     def activate(self, x, activation):
         return x.copy_(self._act(_f(x), activation).to(x.dtype))
 

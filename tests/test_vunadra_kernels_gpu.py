@@ -61,11 +61,6 @@ def test_gelu_gate_and_activation(dtype):
         gu = (2 * torch.randn(T, 2 * inter, generator=g)).to(dtype)
         close(hip.gate_mul(gu.to(DEV), block, "gelu_tanh"), emu.gate_mul(gu, block, "gelu_tanh"), tol)
         close(hip.activate(gu.clone().to(DEV), "gelu_tanh"), emu.activate(gu.clone(), "gelu_tanh"), tol)
-    for T, inter, block in ((3, 40, 8), (17, 96, None), (130, 24, 8), (2, 10, 5)):
-        sums, bias = 2 * torch.randn(T, 2 * inter, generator=g), torch.randn(2 * inter, generator=g)
-        for b in (bias, None):
-            close(hip.gate_mul_sums(sums.to(DEV), None if b is None else b.to(DEV), block, "gelu_tanh"),
-                  emu.gate_mul_sums(sums, b, block, "gelu_tanh"), tol)
     z = torch.linspace(-6, 6, 25, dtype=torch.float64)
     want = 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
     close(emu.activate(z.float().clone(), "gelu_tanh"), want, 1e-6)
