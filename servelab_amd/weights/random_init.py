@@ -57,8 +57,9 @@ class RandomCheckpoint:
     """Seeded random tensors by checkpoint name, drawn on ``device`` when asked
     for: matrices and biases N(0, std), gains 1 + N(0, norm_std).  A tensor's
     values depend on the seed and on its place in ``param_specs`` only.
-    Matrices come in ``dtype``, vectors in float32 (as a loaded checkpoint's
-    vectors are kept by the parts)."""
+    Matrices come in ``dtype``; vectors in float32 (as a loaded checkpoint's
+    vectors are kept by the parts) with values that ``dtype`` holds (as those a
+    checkpoint of that type stores)."""
 
     def __init__(self, param_specs, seed: int, device, dtype: torch.dtype = torch.bfloat16,
                  std: float = 0.02, norm_std: float = 0.05):
@@ -79,7 +80,7 @@ class RandomCheckpoint:
         gen.manual_seed(self.seed * 100003 + self._index[name])
         t = torch.randn(spec.shape, generator=gen, device=self.device, dtype=torch.float32)
         t = t.mul_(self.norm_std).add_(1.0) if spec.init == "gain" else t.mul_(self.std)
-        return t.to(self.dtype) if len(spec.shape) > 1 else t
+        return t.to(self.dtype) if len(spec.shape) > 1 else t.to(self.dtype).float()
 
     def state_dict(self) -> Dict[str, torch.Tensor]:
         return {name: self.get(name) for name in self.specs}
