@@ -186,6 +186,8 @@ def marked_token_model(kind):
     query points at the key that only the token MARK makes, and that token's value is large."""
     if kind == "attention":        # no window: the key is seen 290 tokens later
         layers = [conv_attention(2, 1, 16, 24, 6.0, 3, rot(10000.0, 4), None)]
+    elif kind == "attention_w":    # the same behind a window
+        layers = [conv_attention(2, 1, 16, 24, 6.0, 3, rot(10000.0, 4), None, window=WINDOW)]
     elif kind == "attention_2":
         layers = [key_value_attention(2, 1, 16, 6.0, rot(10000.0, 4), None, window=WINDOW, softcap=25.0)]
     else:
@@ -211,9 +213,12 @@ def marked_token_model(kind):
     w[p + "k"][15, 0] = 4.0                          # channel 15 (not rotated) of the one kv head
     w[p + "q"][15::16] = 0.0
     w[p + "q"][15::16, 1] = 3.0                      # every query head asks for channel 15
-    if kind == "attention":
+    if kind in ("attention", "attention_w"):
         for name in ("q.conv", "k.conv", "v.conv"):  # the marked token's own tap carries it; the other taps stay
             w[p + name][:, -1] = 1.0
+        if kind == "attention_w":                    # (keys and values of the marked token alone, so that the
+            w[p + "k.conv"][:, :-1] = 0.0            # window's edge is one token wide; the queries keep their taps)
+            w[p + "v.conv"][:, :-1] = 0.0
         w[p + "v"][:, 0] = 3.0
     else:
         w[p + "q.norm"][:] = 1.0
@@ -221,7 +226,7 @@ def marked_token_model(kind):
     return cfg, {n: t.to(torch.bfloat16).float() for n, t in w.items()}
 
 
-@pytest.mark.parametrize("kind", ["attention", "attention_2", "latent"])
+@pytest.mark.parametrize("kind", ["attention", "attention_w", "attention_2", "latent"])
 @pytest.mark.parametrize("place", [0, 15, 16, 47, 64, 200])
 def test_a_marked_token_decides_the_logits(tmp_path, kind, place):
     """The marked token at the start, and just before, at and after the borders of pages; in a prompt,
