@@ -9,6 +9,11 @@ row-concatenated weight, the kernel table applies the position encoding (a
 parameter this mixer never looks inside) and writes the pages, and one call
 attends for all sequences of the batch through their block tables.  The
 window (keys p - W < r <= p) is this build's own.
+
+``ProjectionNormAttention`` and ``ShortConvAttention`` are the attention of designs whose softmax
+weights stay float32 and whose keys and values differ in width: a norm over the whole projection,
+biases, keys that serve as values, capped scores and a short convolution before the rotation are
+switches of theirs.
 """
 import math
 

@@ -12,6 +12,10 @@ sublayers read its output; the block returns both outputs as its pending delta
 SandwichBlock: h += Norm1b(Mixer(Norm1(h))); h += Norm2b(FeedForward(Norm2(h))): a norm before and
 after each sublayer.  The norm on an output and the norm before the next sublayer are one kernel
 call, so a block returns its last output with the norm that is still to be applied to it.
+
+StreamReentry: no sublayers; the stream is rewritten as a product of itself and the step's kept
+embedding output side by side, plus a vector of the pass: what a stretch of layers that is walked
+several times starts every pass with.
 """
 from .base import Block, prefixed
 
