@@ -164,7 +164,9 @@ class ProductOps:
         if not isinstance(weight, LinearWeight):
             weight = LinearWeight(weight)
         if isinstance(x, ScaledRows):
-            return self._linear_scaled(x, weight, bias, out_f32, False)
+            if weight.tiled is not None and weight.shape == (weight.shape[0], x.shape[1]):
+                return self._linear_scaled(x, weight, bias, out_f32, False)
+            x = self.finish_scaled_rows(x)      # (a matrix the fused kernels do not take: rows of odd length)
         M, K = x.shape
         N = weight.shape[0]
         if isinstance(x, TiledRows) and not (defer and self.fuse_norms and not out_f32 and N <= 8192):
@@ -360,6 +362,18 @@ class ProductOps:
             self._skinny(xs.x, weight, bias, y, M, N, K, out_f32, gated, scaled=xs, y_tiled=y_tiled)
         return TiledRows(y, (M, N // 2)) if y_tiled else y
 
+    def finish_scaled_rows(self, xs):
+        """Un-normalised rows as plain normed rows in the activation dtype, for a reader whose matrix
+        the fused few-rows kernels do not take: every row times rsqrt(mean x^2 + eps) from the sums
+        of squares the producer left."""
+        x = xs.plain_x()
+        sums = xs.parts.sum(0)                                  # by row of the producer's step
+        if xs.rows is not None:
+            x, sums = x[xs.rows.long()], sums[xs.rows.long()]
+        else:
+            sums = sums[:x.shape[0]]
+        return (x.float() * torch.rsqrt(sums / x.shape[1] + xs.eps)[:, None]).to(self.act_dtype)
+
     def _takes_resident(self, N, K, parts) -> bool:
         """Whether a consumer product runs on the workgroups that stay and walk the tiles
         (x in registers, row scales computed once): matrices with several tiles per CU whose
@@ -387,9 +401,10 @@ class ProductOps:
         if bias is not None:
             self._check(bias, torch.float32, (weight.shape[0],), "bias")
         if isinstance(x, ScaledRows):
-            if block != self.GATE_BLOCK or weight.shape[0] % 16:
-                raise KernelError("un-normalised rows need gate and up in blocks of 8")
-            return self._linear_scaled(x, weight, bias, False, code, y_tiled=_tiled_out)
+            if block == self.GATE_BLOCK and weight.shape[0] % 16 == 0 and weight.tiled is not None:
+                return self._linear_scaled(x, weight, bias, False, code, y_tiled=_tiled_out)
+            x = self.finish_scaled_rows(x)
+            _tiled_out = False
         M, K = x.shape
         N = weight.shape[0]
         if (_tiled_out and M < self._wide_from(K) and M <= self._few_rows_limit(weight)

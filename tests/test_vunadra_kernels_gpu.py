@@ -284,3 +284,36 @@ def test_convolution_inside_the_launch_that_turns_and_stores(dtype, taps):
         rows = hip.short_conv(buf.to(DEV), 0, w.to(DEV), s3, 0, batch_d, True, activation=None)
         q3 = hip.projnorm_rope_store(rows, H, G, D, Dv, dev(qg), dev(kg), 1e-5, rot, tbd, slots.to(DEV), k3, v3, page)
         assert torch.equal(q1, q3) and torch.equal(kd, k3) and torch.equal(vd, v3)
+
+
+def test_rows_a_norm_left_unfinished_reach_a_matrix_of_odd_rows():
+    """A product deferred to the norm that adds it leaves un-normalised rows for the next product to
+    finish; a reader whose matrix has rows of a length the fused kernels do not take gets them finished."""
+    hip, emu = tables(torch.bfloat16)
+    g = torch.Generator().manual_seed(11)
+    for M in (1, 3, 16):
+        x = torch.randn(M, 64, generator=g).to(torch.bfloat16)
+        down = (torch.randn(72, 64, generator=g) / 8).to(torch.bfloat16)
+        head = (torch.randn(100, 72, generator=g) / 8).to(torch.bfloat16)
+        gate_up = (torch.randn(48, 72, generator=g) / 8).to(torch.bfloat16)
+        gain = 1 + 0.3 * torch.randn(72, generator=g)
+        resid = torch.randn(M, 72, generator=g)
+        r2 = resid.clone()
+        want_rows = emu.add_rmsnorm(r2, emu.linear(x, down, None), gain, 1e-5)
+        for reader in ("linear", "gated", "rows"):
+            r1 = resid.clone().to(DEV)
+            d = hip.linear(x.to(DEV), hip.prepare_weight(down.to(DEV), residual_delta=True), None, defer=True)
+            if reader == "rows":
+                rows = torch.tensor([M - 1, 0], dtype=torch.int32)
+                normed = hip.rows_add_rmsnorm(r1, d, rows.to(DEV), gain.to(DEV), 1e-5, fuse=True)
+                got = hip.linear(normed, hip.prepare_weight(head.to(DEV)), None, out_f32=True)
+                close(got, emu.linear(want_rows[rows.long()], head, None, out_f32=True), 2e-2)
+                continue
+            normed = hip.add_rmsnorm(r1, d, gain.to(DEV), 1e-5, fuse=True)
+            close(r1, r2, 1e-2)
+            if reader == "linear":
+                got = hip.linear(normed, hip.prepare_weight(head.to(DEV)), None, out_f32=True)
+                close(got, emu.linear(want_rows, head, None, out_f32=True), 2e-2)
+            else:
+                got = hip.gated_linear(normed, hip.prepare_weight(gate_up.to(DEV)), 8)
+                close(got, emu.gated_linear(want_rows, gate_up, 8), 2e-2)

@@ -84,11 +84,12 @@ def _a():
 def _b():
     # a width that is no multiple of 32; constants that are 1; no loop; no masks (every earlier key); no cap;
     # plain frequencies; part of a head rotated; one choice per token, no expert that hands through; a layer
-    # without a feed-forward; one kv head; a convolution of two taps
+    # without a feed-forward; one kv head; a convolution of two taps; a last feed-forward whose output product
+    # takes the fused few-rows kernel while the head's rows of 72 values do not
     layers = [
         key_value_attention(3, 1, 8, 0.5, rot(500.0, 8), None),
         conv_attention(3, 3, 8, 8, 0.4, 2, rot(100.0, 4), moe(3, 0, 1, 16, 1.0, 1.0)),
-        latent(2, 24, 4, 8, 40, 0.15, 100.0, dense(40)),
+        latent(2, 24, 4, 8, 40, 0.15, 100.0, dense(64)),
     ]
     return config(72, 257, 1e-6, layers)
 
