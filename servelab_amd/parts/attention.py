@@ -118,8 +118,11 @@ class ProjectionNormAttention(Mixer):
     ``projection_norm`` False: q and k go to the rotation as the projection left them (no gains
     in the checkpoint); ``bias`` False: no biases.  ``values`` "keys": there is no value
     projection; a token's values are its keys as the projection left them (with their bias),
-    before norm and rotation.  ``softcap`` c: a scaled score s becomes c tanh(s / c)."""
+    before norm and rotation.  ``softcap`` c: a scaled score s becomes c tanh(s / c).
+    The input goes to nothing but the input product and the output product's result only joins the
+    stream, so in steps of few rows a pre-norm block's norms can run the products around them."""
     graph_safe = True
+    takes_scaled_rows = True
 
     NAMES = {"q": "q", "k": "k", "v": "v", "out": "o", "q_bias": "q.b", "k_bias": "k.b",
              "v_bias": "v.b", "out_bias": "o.b", "q_norm": "q.norm", "k_norm": "k.norm"}
@@ -230,7 +233,7 @@ class ProjectionNormAttention(Mixer):
         attend = (q, 0, H, G, D, Dv, cache.k, cache.v, cache.page_size, group.block_tables, batch, self.scale,
                   self.window)
         attn = ops.window_attention(*attend, softcap=self.softcap) if self.softcap else ops.window_attention(*attend)
-        return ops.linear(attn, self.w_o, self.b_o)
+        return ops.linear(attn, self.w_o, self.b_o, defer=True)
 
 
 class ShortConvAttention(ProjectionNormAttention):
